@@ -1,0 +1,116 @@
+// Shared device-side vocabulary for the gfx950 GEMM-family kernels: vector
+// types, buffer-resource helpers, fp16/bf16 conversion and the XCD-aware
+// workgroup -> output-tile mapping.  gfx950 (MI355X, CDNA4) only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace aitamd {
+
+using f16 = _Float16;
+using bf16 = __bf16;
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define AITAMD_DEVICE __device__ __forceinline__
+
+constexpr int kWaveSize = 64;
+constexpr int kNumXcd = 8;  // MI355X: 8 accelerator dies, one L2 each
+
+// ---------------------------------------------------------------------------
+// Element-type traits: 8-wide operand vector and the 32x32x16 / 16x16x32 MFMA.
+// ---------------------------------------------------------------------------
+template <class T>
+struct ElemTraits;
+
+template <>
+struct ElemTraits<f16> {
+  using vec8 = f16x8;
+  using vec4 = f16x4;
+  static AITAMD_DEVICE f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static AITAMD_DEVICE f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static AITAMD_DEVICE float to_float(f16 v) { return (float)v; }
+  static AITAMD_DEVICE f16 from_float(float v) { return (f16)v; }
+};
+
+template <>
+struct ElemTraits<bf16> {
+  using vec8 = bf16x8;
+  using vec4 = bf16x4;
+  static AITAMD_DEVICE f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static AITAMD_DEVICE f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static AITAMD_DEVICE float to_float(bf16 v) { return (float)v; }
+  static AITAMD_DEVICE bf16 from_float(float v) { return (bf16)v; }
+};
+
+// ---------------------------------------------------------------------------
+// Raw buffer resources.  Loads whose byte offset is >= num_records return 0,
+// which is how every M/N/K tail is zero-filled without branches.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kOobOffset = 0x80000000u;  // >= any num_records we build
+
+AITAMD_DEVICE __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t num_bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, num_bytes, 0x00020000);
+}
+
+AITAMD_DEVICE u32x4 buffer_load_16B(__amdgpu_buffer_rsrc_t r, uint32_t voffset) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, voffset, 0, 0);
+}
+AITAMD_DEVICE u32x2 buffer_load_8B(__amdgpu_buffer_rsrc_t r, uint32_t voffset) {
+  return __builtin_amdgcn_raw_buffer_load_b64(r, voffset, 0, 0);
+}
+AITAMD_DEVICE uint32_t buffer_load_4B(__amdgpu_buffer_rsrc_t r, uint32_t voffset) {
+  return __builtin_amdgcn_raw_buffer_load_b32(r, voffset, 0, 0);
+}
+AITAMD_DEVICE uint16_t buffer_load_2B(__amdgpu_buffer_rsrc_t r, uint32_t voffset) {
+  return __builtin_amdgcn_raw_buffer_load_b16(r, voffset, 0, 0);
+}
+
+// Clamp a 64-bit byte count into the 32-bit num_records field.
+AITAMD_DEVICE uint32_t clamp_records(int64_t bytes) {
+  return bytes <= 0 ? 0u : (bytes >= 0x7fffffffll ? 0x7fffffffu : (uint32_t)bytes);
+}
+
+// ---------------------------------------------------------------------------
+// Workgroup -> tile mapping.  The hardware deals consecutive workgroup ids
+// round-robin over the 8 XCDs; tiles that share an A row-panel or a B
+// column-panel should land on the same XCD so the panel is fetched into one
+// L2 only.  Step 1 gives every XCD a contiguous range of logical tile ids,
+// step 2 walks that range in groups of kGroupM tile-rows, column by column.
+// ---------------------------------------------------------------------------
+template <int kGroupM>
+AITAMD_DEVICE void map_tile(int wg, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int xcd = wg % kNumXcd;
+  const int local = wg / kNumXcd;
+  const int q = total / kNumXcd;
+  const int r = total % kNumXcd;
+  const int id = xcd * q + (xcd < r ? xcd : r) + local;
+  const int group_sz = kGroupM * tiles_n;
+  const int g = id / group_sz;
+  const int first_m = g * kGroupM;
+  const int gm = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
+  const int in_group = id - g * group_sz;
+  tm = first_m + in_group % gm;
+  tn = in_group / gm;
+}
+
+}  // namespace aitamd

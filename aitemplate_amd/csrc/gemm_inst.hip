@@ -1,0 +1,76 @@
+// One translation unit per (epilogue, dtype): compiled repeatedly by the
+// Makefile with -DAITAMD_EPI=<EpilogueId> -DAITAMD_DT=<0 fp16 | 1 bf16>.
+// It instantiates every tile of gemm_tiles.inc for that pair and exports the
+// resulting launcher table under a C symbol the dispatcher looks up.
+#include <mutex>
+
+#include "gemm_host.hpp"
+
+#ifndef AITAMD_EPI
+#error "compile with -DAITAMD_EPI=<id>"
+#endif
+#ifndef AITAMD_DT
+#error "compile with -DAITAMD_DT=<0|1>"
+#endif
+
+namespace aitamd {
+namespace {
+
+#if AITAMD_DT == 0
+using Elem = f16;
+#define AITAMD_DT_NAME "f16"
+#else
+using Elem = bf16;
+#define AITAMD_DT_NAME "bf16"
+#endif
+
+constexpr int kMaxDevices = 64;
+
+template <class Tile>
+hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
+  using Epi = Epilogue<AITAMD_EPI>;
+  auto kernel = gemm_rcr_kernel<Elem, Tile, Epi>;
+  // LDS above 64 KiB has to be opted into once per device.
+  static std::once_flag once[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  hipError_t attr_err = hipSuccess;
+  std::call_once(once[dev % kMaxDevices], [&] {
+    attr_err = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
+  });
+  if (attr_err != hipSuccess) return attr_err;
+
+  GemmParams p = p_in;
+  p.tiles_m = (p.M + Tile::BM - 1) / Tile::BM;
+  p.tiles_n = (p.N + Tile::BN - 1) / Tile::BN;
+  const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+  if (tiles <= 0 || p.batch <= 0) return hipSuccess;
+  if (tiles > 0x7fffffffll) return hipErrorInvalidValue;
+  dim3 grid((unsigned)tiles, (unsigned)(p.batch < 65535 ? p.batch : 65535), 1);
+  hipLaunchKernelGGL(kernel, grid, dim3(Tile::NT), Tile::kLdsBytes, stream, p);
+  return hipGetLastError();
+}
+
+#define AITAMD_STR2(x) #x
+#define AITAMD_STR(x) AITAMD_STR2(x)
+
+const GemmAlgo kAlgos[] = {
+#define AITAMD_GEMM_TILE(BM, BN, BK, WM, WN, KV)                                              \
+  {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_v" #KV,                \
+   BM, BN, BK, GemmTile<BM, BN, BK, WM, WN, KV>::NT, KV, GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes, \
+   &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
+#include "gemm_tiles.inc"
+#undef AITAMD_GEMM_TILE
+};
+
+}  // namespace
+}  // namespace aitamd
+
+#define AITAMD_CAT3(a, b, c) a##b##_##c
+#define AITAMD_TABLE_SYM(e, d) AITAMD_CAT3(aitamd_gemm_table_, e, d)
+
+extern "C" __attribute__((visibility("hidden"))) aitamd::GemmAlgoTable AITAMD_TABLE_SYM(AITAMD_EPI, AITAMD_DT)() {
+  return {aitamd::kAlgos, (int)(sizeof(aitamd::kAlgos) / sizeof(aitamd::kAlgos[0]))};
+}

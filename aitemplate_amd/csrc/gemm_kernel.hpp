@@ -1,0 +1,280 @@
+// RCR GEMM / batched GEMM for gfx950:  C[b][m][n] = epi( sum_k A[b][m][k] * B[b][n][k] ).
+// A is row-major [M,K], B is row-major [N,K] (so both operands are K-contiguous),
+// C is row-major [M,N]; fp16 or bf16 in/out, fp32 accumulate.
+//
+// One workgroup owns a BM x BN output tile.  Per BK-slab of K:
+//   global --(128-bit buffer loads, zero-filled past M/N/K)--> registers
+//          --(128-bit ds_write, XOR-swizzled 16-byte chunks)--> LDS (2 stages)
+//          --(128-bit ds_read)--> v_mfma_f32_32x32x16 operand fragments.
+// The slab for step k+1 is in flight from HBM/L2 while step k is multiplied.
+// The MFMA is issued with the operands swapped (B fragment first), so each lane
+// ends up holding 4 consecutive output columns of one row: bias / residual
+// loads and the output store are 8-byte vector accesses straight from the
+// accumulator registers, with the epilogue evaluated in fp32 in between.
+//
+// Replaces the Composable Kernel device ops the reference instantiates for this
+// family (python/aitemplate/utils/mk_ck_lib/gemm_operation.py:56-66, tile table
+// python/aitemplate/utils/mk_ck_lib/generator.py:517-601,604-785,788-861).
+#pragma once
+
+#include "common.hpp"
+#include "epilogue.hpp"
+
+namespace aitamd {
+
+struct GemmParams {
+  const void* a;
+  const void* b;
+  void* c;
+  const void* bias;  // [N]
+  const void* d0;    // [M, ldd]
+  const void* d1;    // [M, ldd]
+  int32_t M, N, K;
+  int32_t batch;
+  int64_t lda, ldb, ldc, ldd;  // row pitches, in elements
+  int64_t sa, sb, sc, sd;      // batch strides, in elements (0 broadcasts)
+  int32_t tiles_m, tiles_n;
+};
+
+// KVEC = number of K-contiguous elements that may be fetched with one load:
+// 8 -> 128-bit loads (K % 8 == 0, 16-byte aligned rows), 4/2/1 -> narrower
+// pieces for odd K or unaligned views.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int KVEC_>
+struct GemmTile {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_;
+  static constexpr int WGM = WGM_, WGN = WGN_, KVEC = KVEC_;
+  static constexpr int NT = WGM * WGN * kWaveSize;
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;  // per-wave tile
+  static constexpr int MI = WTM / 32, NI = WTN / 32;    // 32x32 MFMA blocks per wave
+  static constexpr int CPR = BK / 8;                    // 16-byte chunks per LDS row
+  static constexpr int RPW = (256 / (BK * 2)) > 0 ? (256 / (BK * 2)) : 1;  // rows per 256-byte bank window
+  static constexpr int A_IT = BM * CPR / NT;
+  static constexpr int B_IT = BN * CPR / NT;
+  static constexpr int ROWS_PER_PASS = NT / CPR;
+  static constexpr int kLdsBytes = 2 * (BM + BN) * BK * 2;
+  static_assert(BM % (WGM * 32) == 0 && BN % (WGN * 32) == 0, "wave tile must be whole MFMA blocks");
+  static_assert(BK % 16 == 0, "BK must be a multiple of the MFMA K");
+  static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "loads must divide evenly");
+  static_assert(NT % CPR == 0, "a load pass must cover whole rows");
+};
+
+// 16-byte chunk `chunk` of LDS row `row` lives at chunk ^ swz(row): any 16
+// consecutive rows read at one logical chunk index touch all 64 banks once.
+template <class Tile>
+AITAMD_DEVICE int lds_chunk_elem(int row, int chunk) {
+  const int swz = (row / Tile::RPW) % Tile::CPR;
+  return row * Tile::BK + ((chunk ^ swz) << 3);
+}
+
+template <class T, class Tile, class Epi>
+__global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) {
+  using Tr = ElemTraits<T>;
+  using vec8 = typename Tr::vec8;
+  constexpr int BM = Tile::BM, BN = Tile::BN, BK = Tile::BK;
+  constexpr int MI = Tile::MI, NI = Tile::NI;
+  constexpr int A_IT = Tile::A_IT, B_IT = Tile::B_IT;
+  constexpr int KVEC = Tile::KVEC;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* const sA = reinterpret_cast<T*>(smem_raw);  // [2][BM*BK]
+  T* const sB = sA + 2 * BM * BK;                // [2][BN*BK]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / Tile::WGN;
+  const int wn = wave % Tile::WGN;
+  const int r32 = lane & 31;
+  const int h = lane >> 5;
+
+  int tm, tn;
+  map_tile<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * BM;
+  const int n0 = tn * BN;
+  const int rows_a = (p.M - m0) < BM ? (p.M - m0) : BM;
+  const int rows_b = (p.N - n0) < BN ? (p.N - n0) : BN;
+
+  // Loop-invariant per-thread load coordinates.
+  const int ld_row = tid / Tile::CPR;
+  const int ld_chunk = tid % Tile::CPR;
+  uint32_t a_off[A_IT], b_off[B_IT];
+  int a_st[A_IT], b_st[B_IT];
+#pragma unroll
+  for (int i = 0; i < A_IT; ++i) {
+    const int row = ld_row + i * Tile::ROWS_PER_PASS;
+    a_off[i] = (uint32_t)(((int64_t)row * p.lda + ld_chunk * 8) * 2);
+    a_st[i] = lds_chunk_elem<Tile>(row, ld_chunk);
+  }
+#pragma unroll
+  for (int i = 0; i < B_IT; ++i) {
+    const int row = ld_row + i * Tile::ROWS_PER_PASS;
+    b_off[i] = (uint32_t)(((int64_t)row * p.ldb + ld_chunk * 8) * 2);
+    b_st[i] = lds_chunk_elem<Tile>(row, ld_chunk);
+  }
+
+  // Loop-invariant fragment read positions (elements), one per 16-wide k step.
+  constexpr int KK = BK / 16;
+  int a_rd[KK], b_rd[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    a_rd[kk] = lds_chunk_elem<Tile>(wm * Tile::WTM + r32, kk * 2 + h);
+    b_rd[kk] = lds_chunk_elem<Tile>(wn * Tile::WTN + r32, kk * 2 + h);
+  }
+
+  const int k_tiles = (p.K + BK - 1) / BK;
+
+  for (int batch = blockIdx.y; batch < p.batch; batch += gridDim.y) {
+    const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)batch * p.sa + (int64_t)m0 * p.lda;
+    const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)batch * p.sb + (int64_t)n0 * p.ldb;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ab, clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
+
+    u32x4 ga[A_IT], gb[B_IT];
+
+    auto load_global = [&](int k0) {
+      if constexpr (KVEC == 8) {
+        const uint32_t kadd = (k0 + ld_chunk * 8 < p.K) ? (uint32_t)(k0 * 2) : kOobOffset;
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) ga[i] = buffer_load_16B(ra, a_off[i] + kadd);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) gb[i] = buffer_load_16B(rb, b_off[i] + kadd);
+      } else {
+        constexpr int PIECES = 8 / KVEC;
+        auto load_pieces = [&](const __amdgpu_buffer_rsrc_t& r, uint32_t base) {
+          union {
+            u32x4 v;
+            uint16_t s[8];
+            uint32_t w[4];
+          } u;
+#pragma unroll
+          for (int j = 0; j < PIECES; ++j) {
+            const int ke = k0 + ld_chunk * 8 + j * KVEC;
+            const uint32_t off = (ke < p.K) ? base + (uint32_t)((k0 + j * KVEC) * 2) : kOobOffset;
+            if constexpr (KVEC == 4) {
+              const u32x2 t = buffer_load_8B(r, off);
+              u.w[2 * j] = t.x;
+              u.w[2 * j + 1] = t.y;
+            } else if constexpr (KVEC == 2) {
+              u.w[j] = buffer_load_4B(r, off);
+            } else {
+              u.s[j] = buffer_load_2B(r, off);
+            }
+          }
+          return u.v;
+        };
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) ga[i] = load_pieces(ra, a_off[i]);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) gb[i] = load_pieces(rb, b_off[i]);
+      }
+    };
+
+    auto store_lds = [&](int stage) {
+      T* dA = sA + stage * BM * BK;
+      T* dB = sB + stage * BN * BK;
+#pragma unroll
+      for (int i = 0; i < A_IT; ++i) *reinterpret_cast<u32x4*>(dA + a_st[i]) = ga[i];
+#pragma unroll
+      for (int i = 0; i < B_IT; ++i) *reinterpret_cast<u32x4*>(dB + b_st[i]) = gb[i];
+    };
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.0f;
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < k_tiles; ++kt) {
+      const int cur = kt & 1;
+      const bool has_next = (kt + 1) < k_tiles;
+      if (has_next) load_global((kt + 1) * BK);
+
+      const T* cA = sA + cur * BM * BK;
+      const T* cB = sB + cur * BN * BK;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        vec8 af[MI], bf[NI];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+          af[mi] = *reinterpret_cast<const vec8*>(cA + a_rd[kk] + mi * 32 * BK);
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+          bf[ni] = *reinterpret_cast<const vec8*>(cB + b_rd[kk] + ni * 32 * BK);
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NI; ++ni)
+            acc[mi][ni] = Tr::mfma32(bf[ni], af[mi], acc[mi][ni]);
+      }
+
+      if (has_next) store_lds(cur ^ 1);
+      __syncthreads();
+    }
+
+    // ---------------- epilogue: registers -> fp32 math -> 8-byte stores -------------
+    T* Cb = reinterpret_cast<T*>(p.c) + (int64_t)batch * p.sc;
+    const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)batch * p.sd : nullptr;
+    const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;
+    const T* bias = reinterpret_cast<const T*>(p.bias);
+
+    bool vec_ok = ((p.N & 3) == 0) && ((p.ldc & 3) == 0) && ((p.sc & 3) == 0) &&
+        ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
+    if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 7) == 0);
+    if (Epi::kNumD >= 1)
+      vec_ok = vec_ok && ((p.ldd & 3) == 0) && ((p.sd & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 7) == 0);
+    if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 7) == 0);
+
+    using vec4 = typename Tr::vec4;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+      const int m = m0 + wm * Tile::WTM + mi * 32 + r32;
+      if (m >= p.M) continue;
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = n0 + wn * Tile::WTN + ni * 32 + g * 8 + h * 4;
+          if (n >= p.N) continue;
+          float v[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] = acc[mi][ni][g * 4 + j];
+          const int64_t c_idx = (int64_t)m * p.ldc + n;
+          const int64_t d_idx = (int64_t)m * p.ldd + n;
+          if (vec_ok) {
+            vec4 bv = {}, d0v = {}, d1v = {};
+            if constexpr (Epi::kHasBias) bv = *reinterpret_cast<const vec4*>(bias + n);
+            if constexpr (Epi::kNumD >= 1) d0v = *reinterpret_cast<const vec4*>(D0b + d_idx);
+            if constexpr (Epi::kNumD >= 2) d1v = *reinterpret_cast<const vec4*>(D1b + d_idx);
+            vec4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              o[j] = Tr::from_float(
+                  Epi::apply(v[j], Tr::to_float(bv[j]), Tr::to_float(d0v[j]), Tr::to_float(d1v[j])));
+            *reinterpret_cast<vec4*>(Cb + c_idx) = o;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              if (n + j < p.N) {
+                float bj = 0.f, d0j = 0.f, d1j = 0.f;
+                if constexpr (Epi::kHasBias) bj = Tr::to_float(bias[n + j]);
+                if constexpr (Epi::kNumD >= 1) d0j = Tr::to_float(D0b[d_idx + j]);
+                if constexpr (Epi::kNumD >= 2) d1j = Tr::to_float(D1b[d_idx + j]);
+                Cb[c_idx + j] = Tr::from_float(Epi::apply(v[j], bj, d0j, d1j));
+              }
+            }
+          }
+        }
+      }
+    }
+    // The next batch iteration overwrites LDS stage 0; every wave has passed the
+    // loop's final barrier after its last LDS read, so no extra barrier is needed.
+  }
+}
+
+}  // namespace aitamd

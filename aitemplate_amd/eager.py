@@ -1,0 +1,114 @@
+"""Direct launches of the GEMM-family kernels on torch device tensors.
+
+Each helper hands raw device pointers, sizes and the current HIP stream to the
+C ABI of the kernel library (``include/aitemplate_amd_kernels.h``); torch is
+used for memory and streams only.  The names and argument order follow the
+reference frontend ops (``ops.gemm_rcr_bias()(a, b, bias)`` etc.,
+python/aitemplate/compiler/ops/gemm_universal/).  There is no fallback path:
+a missing library or a CPU tensor raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _kernels
+
+_TORCH_DTYPE_ID = {torch.float16: 0, torch.bfloat16: 1}
+
+
+def _check(t: Optional[torch.Tensor], name: str, dtype=None):
+    if t is None:
+        return
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor (no CPU path exists)")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name}: dtype {t.dtype} differs from {dtype}")
+
+
+def _stream_ptr() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]) -> Optional[ctypes.c_void_p]:
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _row_pitch(t: torch.Tensor, name: str) -> int:
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise ValueError(f"{name} must be 2-D with a contiguous last dimension")
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], t.stride(0))
+
+
+def gemm(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
+         d0: Optional[torch.Tensor] = None, d1: Optional[torch.Tensor] = None,
+         out: Optional[torch.Tensor] = None, algo: int = -1) -> torch.Tensor:
+    """Run reference op `op` (e.g. "gemm_rcr_bias_gelu"): out = epilogue(a @ b.T, bias, d0, d1).
+
+    `a` may have more than 2 dims; leading dims are flattened into M as the
+    reference does (gemm_rcr.py:51-77).  `algo` = -1 uses the library heuristic,
+    otherwise the instance index (see `_kernels.gemm_algo_names`).
+    """
+    lib = _kernels.load()
+    epi = _kernels.EPILOGUE_OF_OP[op]
+    dtype = a.dtype
+    if dtype not in _TORCH_DTYPE_ID:
+        raise ValueError(f"unsupported dtype {dtype}")
+    for t, n in ((a, "a"), (b, "b"), (bias, "bias"), (d0, "d0"), (d1, "d1"), (out, "out")):
+        _check(t, n, dtype)
+    lead = a.shape[:-1]
+    a2 = a.reshape(-1, a.shape[-1])
+    M, K = a2.shape
+    N = b.shape[0]
+    if b.dim() != 2 or b.shape[1] != K:
+        raise ValueError(f"b must be [N, K={K}], got {tuple(b.shape)}")
+    if out is None:
+        out = torch.empty(*lead, N, dtype=dtype, device=a.device)
+    out2 = out.reshape(-1, N)
+    nres = _kernels.NUM_RESIDUALS_OF_EPILOGUE[epi]
+    if epi != 0 and (bias is None or bias.numel() != N):
+        raise ValueError("bias must be 1-D of size N")
+    d0_2 = d0.reshape(-1, N) if d0 is not None else None
+    d1_2 = d1.reshape(-1, N) if d1 is not None else None
+    if nres >= 1 and (d0_2 is None or d0_2.shape != out2.shape):
+        raise ValueError("d0 must have the output's shape")
+    if nres >= 2 and (d1_2 is None or d1_2.shape != out2.shape):
+        raise ValueError("d1 must have the output's shape")
+    ldd = _row_pitch(d0_2, "d0") if nres >= 1 else N
+    if nres >= 2 and _row_pitch(d1_2, "d1") != ldd:
+        raise ValueError("d0 and d1 must share a row pitch")
+    rc = lib.aitamd_gemm_rcr(epi, _TORCH_DTYPE_ID[dtype], algo, _p(a2), _p(b), _p(bias), _p(d0_2), _p(d1_2),
+                             _p(out2), M, N, K, _row_pitch(a2, "a"), _row_pitch(b, "b"), _row_pitch(out2, "out"),
+                             ldd, _stream_ptr())
+    _kernels.check(rc, op)
+    return out
+
+
+def bmm_rcr(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None, algo: int = -1) -> torch.Tensor:
+    """out[b] = a[b] @ b[b].T with batch broadcast when one operand is 2-D or has batch 1
+    (python/aitemplate/compiler/ops/gemm_universal/bmm.py:72-90)."""
+    lib = _kernels.load()
+    dtype = a.dtype
+    for t, n in ((a, "a"), (b, "b"), (out, "out")):
+        _check(t, n, dtype)
+    a3 = a if a.dim() == 3 else a.unsqueeze(0)
+    b3 = b if b.dim() == 3 else b.unsqueeze(0)
+    if not (a3.is_contiguous() and b3.is_contiguous()):
+        raise ValueError("bmm_rcr operands must be contiguous")
+    B = max(a3.shape[0], b3.shape[0])
+    if a3.shape[0] not in (1, B) or b3.shape[0] not in (1, B):
+        raise ValueError("batch sizes must match or be 1")
+    M, K = a3.shape[1], a3.shape[2]
+    N = b3.shape[1]
+    if b3.shape[2] != K:
+        raise ValueError("K mismatch")
+    if out is None:
+        out = torch.empty(B, M, N, dtype=dtype, device=a.device)
+    sa = 0 if (a3.shape[0] == 1 and B > 1) else M * K
+    sb = 0 if (b3.shape[0] == 1 and B > 1) else N * K
+    rc = lib.aitamd_bmm_rcr(_TORCH_DTYPE_ID[dtype], algo, _p(a3), _p(b3), _p(out), B, M, N, K, K, K, N, sa, sb,
+                            M * N, _stream_ptr())
+    _kernels.check(rc, "bmm_rcr")
+    return out

@@ -1,0 +1,164 @@
+"""Benchmark of the headline configuration: gemm_rcr_bias_gelu, fp16, M=24576 N=3072 K=768
+(BERT-base FFN up-projection), on one MI355X, through the C ABI of the kernel library.
+
+A "step" is one launch of the fused GEMM+bias+GELU over one full-size batch of synthetic
+input that is already resident in HBM.  Operand sets rotate through a pool larger than the
+256 MiB Infinity Cache so every step reads its inputs from HBM.
+
+Prints ONE JSON line:  value = TFLOP/s over the K timed steps (wall clock between two device
+synchronisations);  roofline.achieved = algorithmic FLOPs / average launch duration from HIP
+events recorded around the same K launches on the launch stream;  cpu_baseline = the
+reference tests' PyTorch fp32 expression timed on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+SHAPES = {
+    # name: (op, M, N, K, residuals)
+    "c1": ("gemm_rcr_bias", 256, 1024, 1024, 0),
+    "c2a": ("gemm_rcr_bias_gelu", 24576, 3072, 768, 0),
+    "c2b": ("gemm_rcr_bias_add", 24576, 768, 3072, 1),
+    "c3": ("gemm_rcr_bias_add_add", 12608, 1024, 4096, 2),
+}
+
+
+def _make_pool(torch, op, M, N, K, nres, pool_bytes=600 << 20):
+    set_bytes = 2 * (M * K + N * K + N + (1 + nres) * M * N)
+    sets = max(2, min(16, pool_bytes // set_bytes + 1))
+    g = torch.Generator(device="cuda").manual_seed(1)
+    pool = []
+    for _ in range(sets):
+        x = torch.randn(M, K, device="cuda", generator=g).half()
+        w = (torch.randn(N, K, device="cuda", generator=g) * K ** -0.5).half()
+        b = ((torch.rand(N, device="cuda", generator=g) - 0.5) * 0.2).half()
+        d = [torch.randn(M, N, device="cuda", generator=g).half() for _ in range(nres)]
+        out = torch.empty(M, N, device="cuda", dtype=torch.float16)
+        pool.append((x, w, b, d, out))
+    return pool
+
+
+def time_gemm(torch, eager, name, steps, warmup, algo=-1):
+    op, M, N, K, nres = SHAPES[name]
+    pool = _make_pool(torch, op, M, N, K, nres)
+
+    def step(i):
+        x, w, b, d, out = pool[i % len(pool)]
+        eager.gemm(op, x, w, b, d[0] if nres >= 1 else None, d[1] if nres >= 2 else None, out=out, algo=algo)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ev_ms = e0.elapsed_time(e1)
+    return {"wall_ms_per_step": wall_ms / steps, "event_ms_per_launch": ev_ms / steps,
+            "flops": 2 * M * N * K, "bytes": 2 * (M * K + N * K + N + (1 + nres) * M * N)}
+
+
+def cpu_baseline(torch, max_seconds=20.0):
+    """The oracle expression of the headline config in fp32 on the host cores."""
+    from oracle import oracle
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    op, M, N, K, _ = SHAPES["c2a"]
+    inp = oracle.config_inputs("c2a")
+    x, w, b = inp["x"].float(), inp["w"].float(), inp["bias"].float()
+    times = []
+    t_start = time.perf_counter()
+    for i in range(2 + 5):
+        t0 = time.perf_counter()
+        oracle.torch_gemm(op, x, w, b)
+        dt = time.perf_counter() - t0
+        if i >= 2:
+            times.append(dt)
+        if time.perf_counter() - t_start > max_seconds and len(times) >= 1:
+            break
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": 2 * M * N * K / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"full c2a workload (M={M} N={N} K={K}), fp32 torch F.gelu(F.linear) on CPU, "
+                      f"median of {len(times)} runs after 2 warm-ups, {med * 1e3:.1f} ms each"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--algo", type=int, default=-1, help="kernel instance index (-1: library heuristic)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--all-configs", action="store_true", help="also time the other GEMM configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no exchange step and every GPU box here has one "
+              "GPU; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from aitemplate_amd import _kernels, eager
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    _kernels.load()
+
+    r = time_gemm(torch, eager, "c2a", args.steps, args.warmup, args.algo)
+    tflops = r["flops"] / (r["wall_ms_per_step"] * 1e-3) / 1e12
+    achieved = r["flops"] / (r["event_ms_per_launch"] * 1e-3) / 1e12
+    op, M, N, K, _ = SHAPES["c2a"]
+    algo = args.algo if args.algo >= 0 else _kernels.load().aitamd_gemm_heuristic_algo(3, 0, 1, M, N, K, K, K, 16)
+    line = {
+        "metric": "TFLOP/s + % fp16 MFMA peak, gemm_rcr_bias_gelu M=24576 K=768 N=3072",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(r["wall_ms_per_step"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
+        "config": {"workload": "configs[1]: gemm_rcr_bias_gelu fp16 X[24576,768] W[3072,768] bias[3072], "
+                               "fp32 accumulate, tanh-GELU fused, inputs resident in HBM, rotating operand sets",
+                   "instance": _kernels.gemm_algo_names(3, 0)[algo]},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None},
+    }
+    if args.all_configs:
+        others = {}
+        for name in ("c1", "c2b", "c3"):
+            o = time_gemm(torch, eager, name, max(20, args.steps // 4), max(5, args.warmup // 4))
+            t = o["event_ms_per_launch"] * 1e-3
+            others[name] = {"op": SHAPES[name][0], "ms": round(o["event_ms_per_launch"], 5),
+                            "tflops": round(o["flops"] / t / 1e12, 2), "gbs": round(o["bytes"] / t / 1e9, 1)}
+        line["other_configs"] = others
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,128 @@
+/*
+ * C ABI of libaitemplate_amd_kernels.so: the gfx950 (MI355X) kernels of the
+ * AITemplate ROCm GEMM family and their launch shim.
+ *
+ * These entry points are what the per-op launch functions emitted by the ROCm
+ * GEMM codegen bind to.  In the reference each generated function
+ *     void <op_name>(void* in, void* weight, void* out, [void* bias, void* d0,
+ *                    void* d1,] int64_t* dims..., hipStream_t stream)
+ * (python/aitemplate/backend/rocm/gemm/common.py:107-171, :491-521) builds a
+ * Composable Kernel argument and calls `invoker.Run` (common.py:69-86); here the
+ * same generated function evaluates M/N/K from the dim pointers and calls one
+ * of the launchers below with the algo index its profiler selected.
+ *
+ * Conventions
+ *  - plain pointers and sizes only; all tensor pointers are device pointers;
+ *    `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *  - row-major, K-contiguous operands ("RCR": A[M,K], B[N,K], C[M,N]);
+ *    ld* are row pitches in elements, batch strides are in elements;
+ *  - dtype: 0 = fp16, 1 = bf16 (inputs, residuals and output share it);
+ *    accumulation and the epilogue are fp32;
+ *  - return value 0 on success, non-zero on failure with a thread-local
+ *    message available from aitamd_last_error(); nothing throws across the
+ *    boundary and no entry point synchronises the stream;
+ *  - launchers are re-entrant and stream-ordered: no global mutable state.
+ */
+#ifndef AITEMPLATE_AMD_KERNELS_H_
+#define AITEMPLATE_AMD_KERNELS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AITAMD_API __attribute__((visibility("default")))
+
+/* Epilogue ids == the reference's gemm_flag / element-wise functor table
+ * (python/aitemplate/backend/rocm/gemm/common.py:269-309). */
+enum {
+  AITAMD_EPI_NONE = 0,                  /* gemm_rcr, bmm_rcr          : PassThrough  */
+  AITAMD_EPI_BIAS = 1,                  /* gemm_rcr_bias              : Add          */
+  AITAMD_EPI_BIAS_RELU = 2,             /* gemm_rcr_bias_relu         : AddRelu      */
+  AITAMD_EPI_BIAS_GELU = 3,             /* gemm_rcr_bias_{fast_,}gelu : AddFastGelu  */
+  AITAMD_EPI_BIAS_ADD = 4,              /* gemm_rcr_bias_add          : AddAdd       */
+  AITAMD_EPI_BIAS_ADD_ADD = 5,          /* gemm_rcr_bias_add_add      : AddAddAdd    */
+  AITAMD_EPI_BIAS_ADD_RELU = 6,         /* gemm_rcr_bias_add_relu     : AddAddRelu   */
+  AITAMD_EPI_BIAS_ADD_ADD_RELU = 7,     /* gemm_rcr_bias_add_add_relu : AddAddAddRelu*/
+  AITAMD_EPI_BIAS_SIGMOID = 8,          /* gemm_rcr_bias_sigmoid      : AddSigmoid   */
+  AITAMD_EPI_BIAS_TANH = 9,             /* gemm_rcr_bias_tanh         : AddTanh      */
+  AITAMD_EPI_BIAS_SWISH = 10,           /* gemm_rcr_bias_swish        : AddSwish     */
+  AITAMD_EPI_BIAS_HARDSWISH = 11,       /* gemm_rcr_bias_hardswish    : AddHardswish */
+  AITAMD_EPI_BIAS_MUL = 12,             /* gemm_rcr_bias_mul          : AddMul       */
+  AITAMD_EPI_BIAS_MUL_ADD = 13,         /* gemm_rcr_bias_mul_add      : AddMulAdd    */
+  AITAMD_EPI_BIAS_SIGMOID_MUL = 14,     /* gemm_rcr_bias_sigmoid_mul  : AddSigmoidMul*/
+  AITAMD_EPI_BIAS_SIGMOID_MUL_TANH = 15,/* gemm_rcr_bias_sigmoid_mul_tanh            */
+  AITAMD_EPI_BIAS_MUL_TANH = 16,        /* gemm_rcr_bias_mul_tanh     : AddMulTanh   */
+  AITAMD_NUM_EPILOGUES = 17
+};
+
+enum { AITAMD_F16 = 0, AITAMD_BF16 = 1 };
+
+/* Library version string, e.g. "aitemplate_amd 0.1 gfx950". */
+AITAMD_API const char* aitamd_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). */
+AITAMD_API const char* aitamd_last_error(void);
+
+/* ---- instance ("algo") table: replaces the CK instance manifest the reference
+ * profiler iterates (python/aitemplate/utils/mk_ck_lib/generator.py:517-861,
+ * consumed at python/aitemplate/backend/rocm/gemm/common.py:945-1020). ------- */
+
+/* Number of compiled tile instances for (epilogue, dtype); 0 if none. */
+AITAMD_API int aitamd_gemm_num_algos(int epilogue, int dtype);
+
+/* Name of instance `algo` (stable, used as the profiler's OP:<name>), or NULL. */
+AITAMD_API const char* aitamd_gemm_algo_name(int epilogue, int dtype, int algo);
+
+/* Index of the instance called `name`, or -1. */
+AITAMD_API int aitamd_gemm_find_algo(int epilogue, int dtype, const char* name);
+
+/* 1 if instance `algo` can run this problem (K / pitch / pointer alignment for
+ * its load width), else 0.  `align_bytes` is the smallest power-of-two
+ * alignment shared by the A and B base pointers (pass 16 when unknown-but-
+ * allocator-aligned).  Mirrors the role of CK's IsSupportedArgument
+ * (python/aitemplate/backend/rocm/gemm/common.py:78-82). */
+AITAMD_API int aitamd_gemm_algo_supported(int epilogue, int dtype, int algo,
+                                          int64_t M, int64_t N, int64_t K,
+                                          int64_t lda, int64_t ldb, int align_bytes);
+
+/* Heuristic choice used when no profiling result exists (algo = -1 below);
+ * the counterpart of the reference's select_minimal_algo CI shortcut
+ * (python/aitemplate/backend/rocm/target_def.py:214-234) but shape-aware. */
+AITAMD_API int aitamd_gemm_heuristic_algo(int epilogue, int dtype, int64_t batch,
+                                          int64_t M, int64_t N, int64_t K,
+                                          int64_t lda, int64_t ldb, int align_bytes);
+
+/* ---- launchers ------------------------------------------------------------ */
+
+/* C[m,n] = epilogue( sum_k A[m,k] * B[n,k], bias[n], d0[m,n], d1[m,n] ).
+ * Unused pointers (per the epilogue) may be NULL.  d0/d1 have row pitch ldd.
+ * algo = -1 selects the heuristic instance.  M, N or K equal to 0 is a no-op
+ * (K == 0 still writes epilogue(0, ...), matching an empty sum).
+ * Replaces the generated gemm_rcr* op functions' CK call
+ * (python/aitemplate/backend/rocm/gemm/common.py:132-169). */
+AITAMD_API int aitamd_gemm_rcr(int epilogue, int dtype, int algo,
+                               const void* a, const void* b, const void* bias,
+                               const void* d0, const void* d1, void* c,
+                               int64_t M, int64_t N, int64_t K,
+                               int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                               void* stream);
+
+/* C[b,m,n] = sum_k A[b,m,k] * B[b,n,k]; a batch stride of 0 broadcasts that
+ * operand over the batch (python/aitemplate/compiler/ops/gemm_universal/bmm.py:72-90).
+ * Replaces the generated bmm_rcr op function's CK call
+ * (python/aitemplate/backend/rocm/gemm/bmm_common.py:72-105, bmm_rcr.py:27-182). */
+AITAMD_API int aitamd_bmm_rcr(int dtype, int algo,
+                              const void* a, const void* b, void* c,
+                              int64_t batch, int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldb, int64_t ldc,
+                              int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                              void* stream);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* AITEMPLATE_AMD_KERNELS_H_ */

@@ -1,0 +1,292 @@
+"""TEST INFRASTRUCTURE ONLY — CPU oracle of the AITemplate ROCm GEMM family.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module; nothing under ``aitemplate_amd/`` does.
+
+Two independent restatements are kept side by side:
+
+* ``torch_*`` — the fp32 PyTorch expressions the reference's own unit tests use
+  as their oracle, evaluated on the CPU:
+  ``F.linear`` (tests/unittest/ops/test_gemm_bias.py:69, test_gemm.py),
+  ``relu`` (test_gemm_bias_relu.py:64-65), GELU (test_gemm_rcr_bias_fast_gelu.py:96;
+  the kernel implements the tanh form, see backend/cuda/elementwise/custom_math.cuh:828-851),
+  ``linear + D0 (+ D1)`` (test_gemm_bias_broadcast.py:213-216,372-376),
+  ``bmm(Q, K^T)`` (test_bmm.py:50-51) and
+  ``softmax(Q K^T * scale) V`` with the 0213 permute (test_bmm_softmax_bmm.py:90,111-114).
+* ``c_*`` — the plain-C triple loops of ``oracle/gemm_oracle.c`` (fp32 accumulate,
+  optional reference rounding points), loaded through ctypes.
+
+Parity status: the reference ships no golden vectors for this path (its tests
+compare against PyTorch on a GPU), so every function here is pinned by closed
+forms, invariants and brute force in ``tests/test_oracle.py`` rather than by
+fixtures of the reference.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+from typing import Dict, Optional, Tuple
+
+import numpy as np
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_C_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_c_lib: Optional[ctypes.CDLL] = None
+
+EPILOGUE_ID = {
+    "gemm_rcr": 0, "bmm_rcr": 0, "gemm_rcr_bias": 1, "gemm_rcr_bias_relu": 2, "gemm_rcr_bias_gelu": 3,
+    "gemm_rcr_bias_fast_gelu": 3, "gemm_rcr_bias_add": 4, "gemm_rcr_bias_add_add": 5,
+    "gemm_rcr_bias_add_relu": 6, "gemm_rcr_bias_add_add_relu": 7, "gemm_rcr_bias_sigmoid": 8,
+    "gemm_rcr_bias_tanh": 9, "gemm_rcr_bias_swish": 10, "gemm_rcr_bias_hardswish": 11,
+    "gemm_rcr_bias_mul": 12, "gemm_rcr_bias_mul_add": 13, "gemm_rcr_bias_sigmoid_mul": 14,
+    "gemm_rcr_bias_sigmoid_mul_tanh": 15, "gemm_rcr_bias_mul_tanh": 16,
+}
+
+
+def build_c_oracle() -> str:
+    """Compile oracle/gemm_oracle.c with gcc (a second or two)."""
+    import subprocess
+
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+    return _C_LIB_PATH
+
+
+def c_lib() -> ctypes.CDLL:
+    global _c_lib
+    if _c_lib is None:
+        if not os.path.exists(_C_LIB_PATH):
+            build_c_oracle()
+        lib = ctypes.CDLL(_C_LIB_PATH)
+        i64, i32, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+        lib.oracle_gemm_rcr.restype = i32
+        lib.oracle_gemm_rcr.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i64]
+        lib.oracle_bmm_rcr_epilogue.restype = i32
+        lib.oracle_bmm_rcr_epilogue.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp] + [i64] * 12
+        lib.oracle_bmm_softmax_bmm_permute.restype = i32
+        lib.oracle_bmm_softmax_bmm_permute.argtypes = [i32, i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64,
+                                                       ctypes.c_float, i32]
+        _c_lib = lib
+    return _c_lib
+
+
+# ---------------------------------------------------------------------------
+# torch fp32 expressions (the reference tests' oracle, on the CPU)
+# ---------------------------------------------------------------------------
+def _f(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return None if t is None else t.detach().to("cpu", torch.float32)
+
+
+def torch_epilogue(op: str, y: torch.Tensor, d0=None, d1=None) -> torch.Tensor:
+    """Apply the epilogue named by the reference op to y = X W^T + b (fp32)."""
+    F = torch.nn.functional
+    if op in ("gemm_rcr", "bmm_rcr", "gemm_rcr_bias"):
+        return y
+    if op == "gemm_rcr_bias_relu":
+        return F.relu(y)
+    if op in ("gemm_rcr_bias_gelu", "gemm_rcr_bias_fast_gelu"):
+        return F.gelu(y, approximate="tanh")
+    if op == "gemm_rcr_bias_add":
+        return y + d0
+    if op == "gemm_rcr_bias_add_add":
+        return y + d0 + d1
+    if op == "gemm_rcr_bias_add_relu":
+        return F.relu(y + d0)
+    if op == "gemm_rcr_bias_add_add_relu":
+        return F.relu(y + d0 + d1)
+    if op == "gemm_rcr_bias_sigmoid":
+        return torch.sigmoid(y)
+    if op == "gemm_rcr_bias_tanh":
+        return torch.tanh(y)
+    if op == "gemm_rcr_bias_swish":
+        return y * torch.sigmoid(y)
+    if op == "gemm_rcr_bias_hardswish":
+        return F.hardswish(y)
+    if op == "gemm_rcr_bias_mul":
+        return y * d0
+    if op == "gemm_rcr_bias_mul_add":
+        return y * d0 + d1
+    if op == "gemm_rcr_bias_sigmoid_mul":
+        return torch.sigmoid(y) * d0
+    if op == "gemm_rcr_bias_sigmoid_mul_tanh":
+        return torch.tanh(torch.sigmoid(y) * d0)
+    if op == "gemm_rcr_bias_mul_tanh":
+        return torch.tanh(y * d0)
+    raise KeyError(op)
+
+
+def torch_gemm(op: str, x, w, bias=None, d0=None, d1=None) -> torch.Tensor:
+    """fp32 result of reference op `op`; cast to the input dtype by the caller."""
+    y = torch.nn.functional.linear(_f(x), _f(w), _f(bias) if op != "gemm_rcr" else None)
+    return torch_epilogue(op, y, _f(d0), _f(d1))
+
+
+def torch_bmm_rcr(q, k) -> torch.Tensor:
+    q, k = _f(q), _f(k)
+    if q.dim() == 2:
+        q = q.unsqueeze(0)
+    if k.dim() == 2:
+        k = k.unsqueeze(0)
+    return torch.matmul(q, k.transpose(-1, -2))
+
+
+def torch_bmm_softmax_bmm_permute(q, k, v, scale: float, num_heads: int, causal: bool = False,
+                                  chunk: int = 4) -> torch.Tensor:
+    """softmax(Q K^T * scale) V, output [B/G, M, G, O]; chunked over the batch to bound memory."""
+    q, k, v = _f(q), _f(k), _f(v)
+    B, M, _ = q.shape
+    N, O = v.shape[1], v.shape[2]
+    out = torch.empty(B, M, O, dtype=torch.float32)
+    for s in range(0, B, chunk):
+        att = torch.bmm(q[s:s + chunk], k[s:s + chunk].transpose(1, 2)) * scale
+        if causal:
+            mask = torch.ones(M, N, dtype=torch.bool).tril()
+            att = att.masked_fill(~mask, float("-inf"))
+        att = torch.softmax(att, dim=-1)
+        out[s:s + chunk] = torch.bmm(att, v[s:s + chunk])
+    G = num_heads
+    return out.reshape(B // G, G, M, O).permute(0, 2, 1, 3).contiguous()
+
+
+# ---------------------------------------------------------------------------
+# C restatement through ctypes (inputs: fp16 / bf16 torch CPU tensors)
+# ---------------------------------------------------------------------------
+def _dtype_id(t: torch.Tensor) -> int:
+    return {torch.float16: 0, torch.bfloat16: 1}[t.dtype]
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def c_gemm(op: str, x, w, bias=None, d0=None, d1=None, ref_rounding: bool = False) -> torch.Tensor:
+    x, w = x.cpu().contiguous(), w.cpu().contiguous()
+    bias = None if bias is None else bias.cpu().contiguous()
+    d0 = None if d0 is None else d0.cpu().contiguous()
+    d1 = None if d1 is None else d1.cpu().contiguous()
+    M, K = x.shape
+    N = w.shape[0]
+    out = torch.empty(M, N, dtype=x.dtype)
+    rc = c_lib().oracle_gemm_rcr(EPILOGUE_ID[op], _dtype_id(x), int(ref_rounding), _ptr(x), _ptr(w), _ptr(bias),
+                                 _ptr(d0), _ptr(d1), _ptr(out), M, N, K)
+    assert rc == 0, rc
+    return out
+
+
+def c_bmm_rcr(q, k, ref_rounding: bool = False) -> torch.Tensor:
+    q, k = q.cpu().contiguous(), k.cpu().contiguous()
+    if q.dim() == 2:
+        q = q.unsqueeze(0)
+    if k.dim() == 2:
+        k = k.unsqueeze(0)
+    B = max(q.shape[0], k.shape[0])
+    M, K = q.shape[1], q.shape[2]
+    N = k.shape[1]
+    sa = 0 if q.shape[0] == 1 and B > 1 else M * K
+    sb = 0 if k.shape[0] == 1 and B > 1 else N * K
+    out = torch.empty(B, M, N, dtype=q.dtype)
+    rc = c_lib().oracle_bmm_rcr_epilogue(0, _dtype_id(q), int(ref_rounding), _ptr(q), _ptr(k), None, None, None,
+                                         _ptr(out), B, M, N, K, K, K, N, N, sa, sb, M * N, 0)
+    assert rc == 0, rc
+    return out
+
+
+def c_bmm_softmax_bmm_permute(q, k, v, scale: float, num_heads: int, causal: bool = False,
+                              ref_rounding: bool = False) -> torch.Tensor:
+    q, k, v = q.cpu().contiguous(), k.cpu().contiguous(), v.cpu().contiguous()
+    B, M, K = q.shape
+    N, O = v.shape[1], v.shape[2]
+    G = num_heads
+    out = torch.empty(B // G, M, G, O, dtype=q.dtype)
+    rc = c_lib().oracle_bmm_softmax_bmm_permute(_dtype_id(q), int(ref_rounding), _ptr(q), _ptr(k), _ptr(v),
+                                                _ptr(out), B, M, N, K, O, G, float(scale), int(causal))
+    assert rc == 0, rc
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Seeded synthetic inputs of the five benchmark configurations.
+# Generated on the CPU in fp32 with torch.manual_seed(seed), cast to `dtype`;
+# draw order = order listed.  `scale_down` shrinks M (and the batch) for quick
+# parity cases while keeping every other dimension.
+# ---------------------------------------------------------------------------
+def _u(shape, lo, hi):
+    return torch.rand(*shape) * (hi - lo) + lo
+
+
+def config_inputs(cfg: str, dtype=torch.float16, m_override: Optional[int] = None,
+                  batch_override: Optional[int] = None) -> Dict[str, torch.Tensor]:
+    if cfg == "c1":
+        torch.manual_seed(0)
+        M = m_override or 256
+        d = {"x": _u((M, 1024), -1, 1), "w": _u((1024, 1024), -1, 1), "bias": _u((1024,), -1, 1)}
+    elif cfg == "c2a":
+        torch.manual_seed(1)
+        M = m_override or 24576
+        d = {"x": torch.randn(M, 768), "w": torch.randn(3072, 768) * 768 ** -0.5, "bias": _u((3072,), -0.1, 0.1)}
+    elif cfg == "c2b":
+        torch.manual_seed(2)
+        M = m_override or 24576
+        d = {"x": torch.randn(M, 3072), "w": torch.randn(768, 3072) * 3072 ** -0.5,
+             "bias": _u((768,), -0.1, 0.1), "d0": torch.randn(M, 768)}
+    elif cfg == "c3":
+        torch.manual_seed(3)
+        M = m_override or 12608
+        d = {"x": torch.randn(M, 4096), "w": torch.randn(1024, 4096) * 4096 ** -0.5, "bias": torch.randn(1024),
+             "d0": torch.randn(M, 1024), "d1": torch.randn(M, 1024)}
+    elif cfg == "c4":
+        torch.manual_seed(4)
+        B = batch_override or 768
+        d = {"q": torch.randn(B, 384, 64) / 8.0, "k": torch.randn(B, 384, 64) / 8.0}
+    elif cfg == "c5":
+        torch.manual_seed(5)
+        B = batch_override or 16
+        S = m_override or 4096
+        d = {"q": torch.randn(B, S, 40), "k": torch.randn(B, S, 40), "v": torch.randn(B, S, 40)}
+    else:
+        raise KeyError(cfg)
+    return {k: v.to(dtype) for k, v in d.items()}
+
+
+CONFIG_OP = {
+    "c1": "gemm_rcr_bias",
+    "c2a": "gemm_rcr_bias_gelu",
+    "c2b": "gemm_rcr_bias_add",
+    "c3": "gemm_rcr_bias_add_add",
+    "c4": "bmm_rcr",
+    "c5": "bmm_softmax_bmm_permute",
+}
+C5_HEADS = 8
+C5_SCALE = 40 ** -0.5
+
+
+def config_expected(cfg: str, inp: Dict[str, torch.Tensor]) -> torch.Tensor:
+    """fp32 torch oracle of a configuration (not yet cast to fp16)."""
+    op = CONFIG_OP[cfg]
+    if cfg in ("c1", "c2a", "c2b", "c3"):
+        return torch_gemm(op, inp["x"], inp["w"], inp.get("bias"), inp.get("d0"), inp.get("d1"))
+    if cfg == "c4":
+        return torch_bmm_rcr(inp["q"], inp["k"])
+    return torch_bmm_softmax_bmm_permute(inp["q"], inp["k"], inp["v"], C5_SCALE, C5_HEADS)
+
+
+def config_flops_bytes(cfg: str) -> Tuple[int, int]:
+    """Algorithmic FLOPs and bytes (fp16, every tensor once) of a full-size configuration."""
+    if cfg == "c1":
+        M, N, K, r = 256, 1024, 1024, 0
+    elif cfg == "c2a":
+        M, N, K, r = 24576, 3072, 768, 0
+    elif cfg == "c2b":
+        M, N, K, r = 24576, 768, 3072, 1
+    elif cfg == "c3":
+        M, N, K, r = 12608, 1024, 4096, 2
+    elif cfg == "c4":
+        B, M, N, K = 768, 384, 384, 64
+        return 2 * B * M * N * K, 2 * B * (M * K + N * K + M * N)
+    elif cfg == "c5":
+        B, M, N, K, O = 16, 4096, 4096, 40, 40
+        return 2 * B * M * N * K + 2 * B * M * N * O, 2 * B * (M * K + N * K + N * O + M * O)
+    else:
+        raise KeyError(cfg)
+    return 2 * M * N * K, 2 * (M * K + N * K + N + (1 + r) * M * N)

@@ -1,0 +1,214 @@
+"""Pins of the CPU oracle (no GPU).  The reference holds no golden vectors for the
+GEMM path, so the oracle is pinned by what the mathematics fixes: brute force on
+tiny inputs, special cases that reduce to library routines, and invariants chosen
+so that a dropped term, a transposed operand or a wrong permute fails one of them."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+
+
+def _rand(shape, dtype=torch.float16, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ---- number formats ---------------------------------------------------------
+def test_c_half_conversion_matches_numpy_for_every_half_and_random_floats():
+    lib = oracle.c_lib()
+    # identity GEMM with K=1: c = fp16(a * 1) exercises half->float->half on every finite half
+    bits = np.arange(0, 1 << 16, dtype=np.uint16)
+    finite = bits[((bits & 0x7C00) != 0x7C00) & (bits != 0x8000)]  # 0 + (-0) is +0: skip -0
+    x = torch.from_numpy(finite.view(np.float16).copy()).reshape(-1, 1)
+    one = torch.ones(1, 1, dtype=torch.float16)
+    y = oracle.c_gemm("gemm_rcr", x, one)
+    assert np.array_equal(y.numpy().view(np.uint16).ravel(), finite)
+    # rounding: sums of two halves need a real float->half rounding; numpy is the library routine
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((512, 2)).astype(np.float16)
+    a[:, 0] *= np.float16(1000.0)
+    ones = torch.ones(1, 2, dtype=torch.float16)
+    got = oracle.c_gemm("gemm_rcr", torch.from_numpy(a), ones).numpy().ravel()
+    want = (a[:, 0].astype(np.float32) + a[:, 1].astype(np.float32)).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    # tiny values -> subnormal halves
+    tiny = (rng.standard_normal((512, 2)) * 1e-6).astype(np.float16)
+    got = oracle.c_gemm("gemm_rcr", torch.from_numpy(tiny), ones).numpy().ravel()
+    want = (tiny[:, 0].astype(np.float32) + tiny[:, 1].astype(np.float32)).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_c_bf16_rounding_matches_torch():
+    a = _rand((257, 2), torch.bfloat16, seed=3, scale=50.0)
+    ones = torch.ones(1, 2, dtype=torch.bfloat16)
+    got = oracle.c_gemm("gemm_rcr", a, ones).ravel()
+    want = (a[:, 0].float() + a[:, 1].float()).to(torch.bfloat16)
+    assert torch.equal(got, want)
+
+
+# ---- GEMM: brute force and invariants --------------------------------------
+def _brute_gemm(x, w, bias):
+    M, K = x.shape
+    N = w.shape[0]
+    out = [[0.0] * N for _ in range(M)]
+    for m in range(M):
+        for n in range(N):
+            s = 0.0
+            for k in range(K):
+                s += float(x[m, k]) * float(w[n, k])
+            out[m][n] = s + (float(bias[n]) if bias is not None else 0.0)
+    return torch.tensor(out, dtype=torch.float64)
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 5, 7), (16, 16, 16), (1, 9, 4), (8, 1, 3)])
+def test_gemm_matches_brute_force(M, N, K):
+    x, w, b = _rand((M, K), seed=1), _rand((N, K), seed=2), _rand((N,), seed=3)
+    want = _brute_gemm(x, w, b)
+    got_t = oracle.torch_gemm("gemm_rcr_bias", x, w, b).double()
+    got_c = oracle.c_gemm("gemm_rcr_bias", x, w, b).double()
+    assert torch.allclose(got_t, want, atol=1e-4, rtol=1e-5)
+    assert torch.allclose(got_c, want, atol=1e-2, rtol=1e-3)  # rounded to fp16
+    # a transposed W would fail here: W is not square and not symmetric
+    want_nb = _brute_gemm(x, w, None)
+    assert torch.allclose(oracle.torch_gemm("gemm_rcr", x, w).double(), want_nb, atol=1e-4, rtol=1e-5)
+
+
+def test_gemm_identity_weight_and_zero_input():
+    x, b = _rand((12, 32), seed=4), _rand((32,), seed=5)
+    eye = torch.eye(32, dtype=torch.float16)
+    for f in (oracle.torch_gemm, oracle.c_gemm):
+        y = f("gemm_rcr_bias", x, eye, b).float()
+        assert torch.allclose(y, (x.float() + b.float()), atol=2e-3, rtol=1e-3)
+        z = f("gemm_rcr_bias", torch.zeros_like(x), _rand((8, 32), seed=6), b[:8]).float()
+        assert torch.allclose(z, b[:8].float().expand(12, 8), atol=0, rtol=0)
+
+
+def test_gelu_closed_form_and_identities():
+    x = torch.linspace(-8, 8, 4001)
+    u = math.sqrt(2 / math.pi) * (x + 0.044715 * x ** 3)
+    closed = 0.5 * x * (1 + torch.tanh(u))
+    lib = torch.nn.functional.gelu(x, approximate="tanh")
+    assert torch.allclose(closed, lib, atol=1e-6)
+    # sigmoid form with the reference's rounded constants (custom_math.cuh:828-851)
+    sig = x / (1 + torch.exp(-2 * x * (0.797885 + 0.035677 * x * x)))
+    assert (sig - lib).abs().max() < 2e-5
+    # erf GELU (what the reference's ROCm test compares against) is within 5e-4 of it... loosely 1e-3
+    assert (torch.nn.functional.gelu(x) - lib).abs().max() < 1e-3
+
+
+EPILOGUE_CASES = ["gemm_rcr", "gemm_rcr_bias", "gemm_rcr_bias_relu", "gemm_rcr_bias_gelu", "gemm_rcr_bias_add",
+                  "gemm_rcr_bias_add_add", "gemm_rcr_bias_add_relu", "gemm_rcr_bias_add_add_relu",
+                  "gemm_rcr_bias_sigmoid", "gemm_rcr_bias_tanh", "gemm_rcr_bias_swish", "gemm_rcr_bias_hardswish",
+                  "gemm_rcr_bias_mul", "gemm_rcr_bias_mul_add", "gemm_rcr_bias_sigmoid_mul",
+                  "gemm_rcr_bias_sigmoid_mul_tanh", "gemm_rcr_bias_mul_tanh"]
+
+
+@pytest.mark.parametrize("op", EPILOGUE_CASES)
+def test_c_and_torch_restatements_agree(op):
+    M, N, K = 33, 20, 48
+    x, w, b = _rand((M, K), seed=7), _rand((N, K), seed=8, scale=K ** -0.5), _rand((N,), seed=9)
+    d0, d1 = _rand((M, N), seed=10), _rand((M, N), seed=11)
+    want = oracle.torch_gemm(op, x, w, b, d0, d1)
+    got = oracle.c_gemm(op, x, w, b, d0, d1).float()
+    assert torch.allclose(got, want, atol=2e-3, rtol=2e-3), (got - want).abs().max()
+    # the reference's rounding points move the result by a few fp16 ulps only
+    got_ref = oracle.c_gemm(op, x, w, b, d0, d1, ref_rounding=True).float()
+    assert torch.allclose(got_ref, want, atol=1e-2, rtol=1e-2)
+
+
+def test_epilogue_terms_are_all_present():
+    # each residual / bias term changes the output: a dropped term fails
+    M, N, K = 4, 8, 8
+    x, w = _rand((M, K), seed=1), _rand((N, K), seed=2)
+    b = torch.full((N,), 2.0, dtype=torch.float16)
+    d0 = torch.full((M, N), 16.0, dtype=torch.float16)
+    d1 = torch.full((M, N), 128.0, dtype=torch.float16)
+    base = oracle.torch_gemm("gemm_rcr", x, w)
+    for f in (oracle.torch_gemm, lambda *a: oracle.c_gemm(*a).float()):
+        assert torch.allclose(f("gemm_rcr_bias", x, w, b) - base, torch.full((M, N), 2.0), atol=3e-2)
+        assert torch.allclose(f("gemm_rcr_bias_add", x, w, b, d0) - base, torch.full((M, N), 18.0), atol=3e-2)
+        assert torch.allclose(f("gemm_rcr_bias_add_add", x, w, b, d0, d1) - base, torch.full((M, N), 146.0),
+                              atol=2e-1)
+
+
+# ---- bmm --------------------------------------------------------------------
+def test_bmm_rcr_brute_force_and_broadcast():
+    q, k = _rand((3, 4, 6), seed=1), _rand((3, 5, 6), seed=2)
+    want = torch.einsum("bmk,bnk->bmn", q.double(), k.double())
+    assert torch.allclose(oracle.torch_bmm_rcr(q, k).double(), want, atol=1e-5)
+    assert torch.allclose(oracle.c_bmm_rcr(q, k).double(), want, atol=1e-2, rtol=1e-2)
+    # broadcast of a batch-1 / 2-D operand
+    k1 = k[:1]
+    want_b = torch.einsum("bmk,nk->bmn", q.double(), k1[0].double())
+    assert torch.allclose(oracle.torch_bmm_rcr(q, k1).double(), want_b, atol=1e-5)
+    assert torch.allclose(oracle.c_bmm_rcr(q, k1[0]).double(), want_b, atol=1e-2, rtol=1e-2)
+
+
+# ---- attention --------------------------------------------------------------
+def _brute_attention(q, k, v, scale, G, causal=False):
+    B, M, K = q.shape
+    N, O = v.shape[1], v.shape[2]
+    out = torch.zeros(B // G, M, G, O, dtype=torch.float64)
+    for b in range(B):
+        for m in range(M):
+            n_end = min(m + 1, N) if causal else N
+            s = [sum(float(q[b, m, kk]) * float(k[b, n, kk]) for kk in range(K)) * scale for n in range(n_end)]
+            mx = max(s)
+            e = [math.exp(t - mx) for t in s]
+            z = sum(e)
+            for o in range(O):
+                out[b // G, m, b % G, o] = sum(e[n] * float(v[b, n, o]) for n in range(n_end)) / z
+    return out
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_brute_force(causal):
+    B, M, N, K, O, G = 4, 5, 7, 3, 6, 2
+    if causal:
+        N = M
+    q, k, v = _rand((B, M, K), seed=1), _rand((B, N, K), seed=2), _rand((B, N, O), seed=3)
+    want = _brute_attention(q, k, v, 0.37, G, causal)
+    got_t = oracle.torch_bmm_softmax_bmm_permute(q, k, v, 0.37, G, causal).double()
+    got_c = oracle.c_bmm_softmax_bmm_permute(q, k, v, 0.37, G, causal).double()
+    assert got_t.shape == (B // G, M, G, O)
+    assert torch.allclose(got_t, want, atol=1e-5)
+    assert torch.allclose(got_c, want, atol=2e-3, rtol=2e-3)
+
+
+def test_attention_invariants():
+    B, M, N, K, O, G = 8, 16, 24, 40, 40, 4
+    q, k, v = _rand((B, M, K), seed=1), _rand((B, N, K), seed=2), _rand((B, N, O), seed=3)
+    for f in (oracle.torch_bmm_softmax_bmm_permute, lambda *a: oracle.c_bmm_softmax_bmm_permute(*a).float()):
+        # rows of P sum to one: constant V -> constant output
+        vc = torch.full_like(v, 0.75)
+        assert torch.allclose(f(q, k, vc, 0.2, G), torch.full((B // G, M, G, O), 0.75), atol=1e-3)
+        # Q = 0 -> uniform attention -> column mean of V
+        out = f(torch.zeros_like(q), k, v, 0.2, G)
+        mean = v.float().mean(dim=1)  # [B, O]
+        want = mean.reshape(B // G, G, 1, O).permute(0, 2, 1, 3).expand(B // G, M, G, O)
+        assert torch.allclose(out, want, atol=2e-3)
+        # permutation: V[b] = b (one value per batch) lands at [b // G, :, b % G, :]
+        vb = torch.arange(B, dtype=torch.float32).reshape(B, 1, 1).expand(B, N, O).to(torch.float16)
+        out = f(q, k, vb, 0.2, G)
+        for b in range(B):
+            assert torch.allclose(out[b // G, :, b % G, :], torch.full((M, O), float(b)), atol=1e-2)
+
+
+def test_config_generators_and_work_counts():
+    inp = oracle.config_inputs("c1")
+    assert inp["x"].shape == (256, 1024) and inp["w"].shape == (1024, 1024) and inp["bias"].shape == (1024,)
+    assert float(inp["x"].float().abs().max()) <= 1.0
+    # determinism
+    again = oracle.config_inputs("c1")
+    assert torch.equal(inp["x"], again["x"])
+    assert oracle.config_flops_bytes("c1") == (536870912, 3147776)
+    assert oracle.config_flops_bytes("c2a") == (115964116992, 193468416)
+    assert oracle.config_flops_bytes("c2b") == (115964116992, 231212544)
+    assert oracle.config_flops_bytes("c3") == (105763569664, 189138944)
+    assert oracle.config_flops_bytes("c4") == (14495514624, 301989888)
+    assert oracle.config_flops_bytes("c5") == (42949672960, 20971520)
+    small = oracle.config_inputs("c3", m_override=200)
+    assert small["x"].shape == (200, 4096) and small["d1"].shape == (200, 1024)
