@@ -17,6 +17,8 @@ struct GemmAlgo {
   int threads;
   int kvec;
   int lds_bytes;
+  int wgs_per_cu;  // workgroups of this instance one CU holds at once
+  int direct_lds;  // 1: direct-to-LDS ring pipeline, 0: register-staged loads
   hipError_t (*launch)(const GemmParams& p, hipStream_t stream);
 };
 

@@ -5,6 +5,7 @@
 #include <mutex>
 
 #include "gemm_host.hpp"
+#include "gemm_kernel_dma.hpp"
 
 #ifndef AITAMD_EPI
 #error "compile with -DAITAMD_EPI=<id>"
@@ -26,10 +27,21 @@ using Elem = bf16;
 
 constexpr int kMaxDevices = 64;
 
+using Epi = Epilogue<AITAMD_EPI>;
+
+template <class Tile>
+struct KernelOf {
+  static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi>;
+};
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
+struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>> {
+  static constexpr auto value =
+      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, Epi>;
+};
+
 template <class Tile>
 hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
-  using Epi = Epilogue<AITAMD_EPI>;
-  auto kernel = gemm_rcr_kernel<Elem, Tile, Epi>;
+  auto kernel = KernelOf<Tile>::value;
   // LDS above 64 KiB has to be opted into once per device.
   static std::once_flag once[kMaxDevices];
   int dev = 0;
@@ -53,6 +65,24 @@ hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Workgroups one CU can hold: limited by LDS (160 KiB) and by the register file
+// (512 VGPRs per SIMD lane shared by the waves of a SIMD).
+constexpr int kLdsPerCu = 160 * 1024;
+constexpr int staged_wgs_per_cu(int bm, int bn, int nt, int lds) {
+  const int acc = bm * bn / nt;                       // fp32 accumulators per lane
+  const int regs = acc + 96;                          // plus staging / fragments / addresses
+  const int waves_per_simd = 512 / regs > 0 ? 512 / regs : 1;
+  const int by_regs = waves_per_simd * 4 / (nt / 64) > 0 ? waves_per_simd * 4 / (nt / 64) : 1;
+  const int by_lds = kLdsPerCu / lds > 0 ? kLdsPerCu / lds : 1;
+  return by_regs < by_lds ? by_regs : by_lds;
+}
+constexpr int dma_wgs_per_cu(int nt, int occ, int lds) {
+  const int waves_per_wg_per_simd = nt / 64 / 4 > 0 ? nt / 64 / 4 : 1;
+  const int by_regs = occ / waves_per_wg_per_simd > 0 ? occ / waves_per_wg_per_simd : 1;
+  const int by_lds = kLdsPerCu / lds > 0 ? kLdsPerCu / lds : 1;
+  return by_regs < by_lds ? by_regs : by_lds;
+}
+
 #define AITAMD_STR2(x) #x
 #define AITAMD_STR(x) AITAMD_STR2(x)
 
@@ -60,9 +90,20 @@ const GemmAlgo kAlgos[] = {
 #define AITAMD_GEMM_TILE(BM, BN, BK, WM, WN, KV)                                              \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_v" #KV,                \
    BM, BN, BK, GemmTile<BM, BN, BK, WM, WN, KV>::NT, KV, GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes, \
-   &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
+   staged_wgs_per_cu(BM, BN, GemmTile<BM, BN, BK, WM, WN, KV>::NT,                                  \
+                     GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes),                                  \
+   0, &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
+#define AITAMD_GEMM_TILE_DMA(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX)                                 \
+  {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
+   "_c" #AUX,                                                                                              \
+   BM, BN, BK, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::NT, 8,                             \
+   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kLdsBytes,                                     \
+   dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::NT, OCC,                        \
+                  GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kLdsBytes),                      \
+   1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>},
 #include "gemm_tiles.inc"
 #undef AITAMD_GEMM_TILE
+#undef AITAMD_GEMM_TILE_DMA
 };
 
 }  // namespace

@@ -59,19 +59,22 @@ def gemm(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor]
     for t, n in ((a, "a"), (b, "b"), (bias, "bias"), (d0, "d0"), (d1, "d1"), (out, "out")):
         _check(t, n, dtype)
     lead = a.shape[:-1]
-    a2 = a.reshape(-1, a.shape[-1])
-    M, K = a2.shape
+    K = a.shape[-1]
+    M = 1
+    for d in lead:
+        M *= d
+    a2 = a.reshape(M, K)
     N = b.shape[0]
     if b.dim() != 2 or b.shape[1] != K:
         raise ValueError(f"b must be [N, K={K}], got {tuple(b.shape)}")
     if out is None:
         out = torch.empty(*lead, N, dtype=dtype, device=a.device)
-    out2 = out.reshape(-1, N)
+    out2 = out.reshape(M, N)
     nres = _kernels.NUM_RESIDUALS_OF_EPILOGUE[epi]
     if epi != 0 and (bias is None or bias.numel() != N):
         raise ValueError("bias must be 1-D of size N")
-    d0_2 = d0.reshape(-1, N) if d0 is not None else None
-    d1_2 = d1.reshape(-1, N) if d1 is not None else None
+    d0_2 = d0.reshape(M, N) if d0 is not None else None
+    d1_2 = d1.reshape(M, N) if d1 is not None else None
     if nres >= 1 and (d0_2 is None or d0_2.shape != out2.shape):
         raise ValueError("d0 must have the output's shape")
     if nres >= 2 and (d1_2 is None or d1_2.shape != out2.shape):
