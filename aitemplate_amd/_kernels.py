@@ -57,6 +57,7 @@ EXPORTED_SYMBOLS = [
     "aitamd_gemm_heuristic_algo",
     "aitamd_gemm_rcr",
     "aitamd_bmm_rcr",
+    "aitamd_bmm_softmax_bmm_permute",
 ]
 
 _lock = threading.Lock()
@@ -98,6 +99,9 @@ def load() -> ctypes.CDLL:
         lib.aitamd_gemm_rcr.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]
         lib.aitamd_bmm_rcr.restype = i32
         lib.aitamd_bmm_rcr.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
+        lib.aitamd_bmm_softmax_bmm_permute.restype = i32
+        lib.aitamd_bmm_softmax_bmm_permute.argtypes = [i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64,
+                                                       ctypes.c_float, i32, vp]
         _lib = lib
         return lib
 

@@ -1,0 +1,100 @@
+// C ABI launcher of the fused attention kernel (bmm_softmax_bmm_permute).
+#include <mutex>
+
+#include "../../include/aitemplate_amd_kernels.h"
+#include "attention_kernel.hpp"
+#include "errors.hpp"
+
+namespace aitamd {
+namespace {
+
+constexpr int kMaxDevices = 64;
+
+template <class T, int KS, int OT, bool VEC>
+hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
+  using Tile = AttnTile<KS, OT>;
+  auto kernel = attention_kernel<T, Tile, VEC>;
+  static std::once_flag once[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  hipError_t attr_err = hipSuccess;
+  std::call_once(once[dev % kMaxDevices], [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
+  });
+  if (attr_err != hipSuccess) return attr_err;
+  const int64_t m_tiles = (p.M + Tile::BM - 1) / Tile::BM;
+  dim3 grid((unsigned)m_tiles, (unsigned)(p.B < 65535 ? p.B : 65535), 1);
+  hipLaunchKernelGGL(kernel, grid, dim3(Tile::NT), Tile::kLdsBytes, stream, p);
+  return hipGetLastError();
+}
+
+typedef hipError_t (*AttnLaunch)(const AttnParams&, hipStream_t);
+
+template <class T, bool VEC>
+AttnLaunch pick(int ks, int ot) {
+#define AITAMD_ATTN_CASE(KS, OT) \
+  if (ks <= KS && ot <= OT) return &launch_attention<T, KS, OT, VEC>;
+  // smallest padded head dims first; (K <= 16 KS, O <= 32 OT)
+  AITAMD_ATTN_CASE(2, 1)
+  AITAMD_ATTN_CASE(3, 2)
+  AITAMD_ATTN_CASE(4, 2)
+  AITAMD_ATTN_CASE(4, 4)
+  AITAMD_ATTN_CASE(6, 3)
+  AITAMD_ATTN_CASE(8, 4)
+#undef AITAMD_ATTN_CASE
+  return nullptr;
+}
+
+float round_to_elem(float x, int dtype) {
+  if (dtype == 0) return (float)(_Float16)x;
+  return (float)(__bf16)x;
+}
+
+}  // namespace
+}  // namespace aitamd
+
+using namespace aitamd;
+
+extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const void* k, const void* v, void* out,
+                                              int64_t B, int64_t M, int64_t N, int64_t K, int64_t O, int64_t G,
+                                              float scale, int causal, void* stream) {
+  if (dtype != 0 && dtype != 1) return fail("aitamd_bmm_softmax_bmm_permute: bad dtype %d", dtype);
+  if (B < 0 || M < 0 || N < 0 || K < 0 || O < 0) return fail("aitamd_bmm_softmax_bmm_permute: negative dimension");
+  if (G <= 0 || (B % G) != 0) return fail("aitamd_bmm_softmax_bmm_permute: batch %lld is not a multiple of heads %lld",
+                                          (long long)B, (long long)G);
+  if (B == 0 || M == 0 || O == 0) return 0;
+  if (B > 0x7fffffffll || M > 0x7fffffffll || N > 0x7fffffffll) return fail("aitamd_bmm_softmax_bmm_permute: dimension too large");
+  if (K > 128 || O > 128) return fail("aitamd_bmm_softmax_bmm_permute: head dims above 128 are not supported (K=%lld O=%lld)",
+                                      (long long)K, (long long)O);
+  if (!out || (N > 0 && (!q || !k || !v))) return fail("aitamd_bmm_softmax_bmm_permute: null pointer");
+  AttnParams p{};
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.out = out;
+  p.B = (int32_t)B;
+  p.M = (int32_t)M;
+  p.N = (int32_t)N;
+  p.K = (int32_t)K;
+  p.O = (int32_t)O;
+  p.G = (int32_t)G;
+  // the reference hands alpha to its kernel in the element type
+  // (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:47-51)
+  p.scale_log2e = round_to_elem(scale, dtype) * 1.4426950408889634f;
+  p.causal = causal ? 1 : 0;
+  const int ks = (int)((K + 15) / 16) > 0 ? (int)((K + 15) / 16) : 1;
+  const int ot = (int)((O + 31) / 32);
+  const bool vec = (K % 8 == 0) && (O % 8 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15) == 0) &&
+      ((reinterpret_cast<uintptr_t>(k) & 15) == 0) && ((reinterpret_cast<uintptr_t>(v) & 15) == 0);
+  AttnLaunch fn = nullptr;
+  if (dtype == 0)
+    fn = vec ? pick<f16, true>(ks, ot) : pick<f16, false>(ks, ot);
+  else
+    fn = vec ? pick<bf16, true>(ks, ot) : pick<bf16, false>(ks, ot);
+  if (!fn) return fail("aitamd_bmm_softmax_bmm_permute: no instance for K=%lld O=%lld", (long long)K, (long long)O);
+  const hipError_t e = fn(p, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail("aitamd_bmm_softmax_bmm_permute: launch failed: %s", hipGetErrorString(e));
+  return 0;
+}

@@ -1,0 +1,315 @@
+// Fused  out = softmax(scale * Q K^T) V  with the [B,M,O] -> [B/G, M, G, O] permute
+// folded into the store (bmm_softmax_bmm_permute), gfx950.
+//
+// The score matrix never leaves the chip.  One wave owns 32 query rows and walks
+// the keys/values in blocks of 32; a workgroup of 4 waves shares each 64-row
+// K / V tile through LDS.
+//
+//  * S^T = K Q^T is computed with v_mfma_f32_32x32x16 (K tile rows as the A
+//    operand, the wave's Q rows - kept in registers for the whole kernel - as
+//    the B operand).  In the accumulator layout of the transposed product a
+//    lane holds 16 keys of ONE query row, so the online-softmax state (running
+//    max, running sum, rescale factor) is one scalar per lane and the row
+//    reductions are 15 in-lane ops plus a single v_permlane32_swap.
+//  * The probabilities, rounded to the element type, are already laid out as the
+//    B operand of the second MFMA  O^T = V^T P^T : no shuffle, no LDS round trip.
+//  * V stays row-major [key][o] in LDS exactly as it sits in memory; the V^T
+//    operand fragments are fetched with ds_read_b64_tr_b16 (LDS transpose read).
+//  * head dims that are not MFMA multiples (40) are zero-padded inside the LDS
+//    tiles only: K to 16*KS columns, V to 32*OT columns.
+//
+// Replaces DeviceBatchedGemmSoftmaxGemmPermute_Xdl_CShuffle as instantiated by
+// the reference (python/aitemplate/utils/mk_ck_lib/gemm_operation.py:64,415-424;
+// arguments python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:84-110).
+#pragma once
+
+#include "common.hpp"
+
+namespace aitamd {
+
+struct AttnParams {
+  const void* q;  // [B, M, K]
+  const void* k;  // [B, N, K]
+  const void* v;  // [B, N, O]
+  void* out;      // [B / G, M, G, O]
+  int32_t B, M, N, K, O, G;
+  float scale_log2e;  // scale (already rounded to the element type) * log2(e)
+  int32_t causal;
+};
+
+template <int KS_, int OT_>
+struct AttnTile {
+  static constexpr int KS = KS_;          // K padded to 16 * KS
+  static constexpr int OT = OT_;          // O padded to 32 * OT
+  static constexpr int KP = 16 * KS;
+  static constexpr int OP = 32 * OT;
+  static constexpr int BM = 128;          // query rows per workgroup (4 waves x 32)
+  static constexpr int BN = 64;           // keys per LDS tile
+  static constexpr int NT = 256;
+  static constexpr int K_PITCH = KP + 8;  // halves; keeps 16 consecutive rows on distinct banks
+  static constexpr int V_PITCH = OP + 8;
+  static constexpr int K_CHUNKS = BN * KP / 8;  // 16-byte chunks per tile (pads included)
+  static constexpr int V_CHUNKS = BN * OP / 8;
+  static constexpr int K_IT = (K_CHUNKS + NT - 1) / NT;
+  static constexpr int V_IT = (V_CHUNKS + NT - 1) / NT;
+  static constexpr int kLdsBytes = 2 * BN * (K_PITCH + V_PITCH) * 2;
+};
+
+// LDS transpose read: 4 x 16-bit per lane, gathered across the 16 lanes of a block
+template <class T>
+struct AttnVec;
+template <>
+struct AttnVec<f16> {
+  typedef __fp16 raw4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+  static AITAMD_DEVICE f16x4 tr_read(const f16* p) {
+    const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((__attribute__((address_space(3))) raw4*)p);
+    return __builtin_bit_cast(f16x4, r);
+  }
+};
+template <>
+struct AttnVec<bf16> {
+  typedef __bf16 raw4 __attribute__((__vector_size__(4 * sizeof(__bf16))));
+  static AITAMD_DEVICE bf16x4 tr_read(const bf16* p) {
+    const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) raw4*)p);
+    return __builtin_bit_cast(bf16x4, r);
+  }
+};
+
+AITAMD_DEVICE float max_across_halves(float x) {
+  // lane l and lane l^32 hold the two halves of one query row
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+AITAMD_DEVICE float sum_across_halves(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// VEC: K and O are multiples of 8 and all base pointers 16-byte aligned -> 128-bit
+// loads; otherwise elements are gathered one by one (slow, any shape).
+template <class T, class Tile, bool VEC>
+__global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams p) {
+  using Tr = ElemTraits<T>;
+  using vec8 = typename Tr::vec8;
+  using vec4 = typename Tr::vec4;
+  constexpr int KS = Tile::KS, OT = Tile::OT, KP = Tile::KP, OP = Tile::OP;
+  constexpr int BN = Tile::BN, KPI = Tile::K_PITCH, VPI = Tile::V_PITCH;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* const sK = reinterpret_cast<T*>(smem_raw);  // [2][BN][K_PITCH]
+  T* const sV = sK + 2 * BN * KPI;               // [2][BN][V_PITCH]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int r32 = lane & 31;
+  const int h = lane >> 5;
+  const int m0 = blockIdx.x * Tile::BM;
+  const int q_row = m0 + wave * 32 + r32;  // this lane's query row
+
+  for (int b = blockIdx.y; b < p.B; b += gridDim.y) {
+    const T* Qb = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.M * p.K;
+    const T* Kb = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.N * p.K;
+    const T* Vb = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.N * p.O;
+
+    // ---- Q fragments (B operand of S^T = K Q^T): lane (q = r32, k = 16 ks + 8 h + j)
+    vec8 qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int k0 = ks * 16 + h * 8;
+      vec8 v = {};
+      if (q_row < p.M) {
+        if (VEC) {
+          if (k0 < p.K) v = *reinterpret_cast<const vec8*>(Qb + (int64_t)q_row * p.K + k0);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (k0 + j < p.K) v[j] = Qb[(int64_t)q_row * p.K + k0 + j];
+        }
+      }
+      qf[ks] = v;
+    }
+
+    // ---- tile loaders: global -> registers -> LDS, zero-filled past N / K / O
+    u32x4 kreg[Tile::K_IT], vreg[Tile::V_IT];
+    auto gather = [&](const T* base, int row, int col, int rows, int cols) -> u32x4 {
+      union {
+        u32x4 v;
+        T e[8];
+      } u;
+      u.v = u32x4{0, 0, 0, 0};
+      if (row < rows) {
+        if (VEC) {
+          if (col < cols) u.v = *reinterpret_cast<const u32x4*>(base + (int64_t)row * cols + col);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (col + j < cols) u.e[j] = base[(int64_t)row * cols + col + j];
+        }
+      }
+      return u.v;
+    };
+    auto load_tiles = [&](int n0) {
+#pragma unroll
+      for (int i = 0; i < Tile::K_IT; ++i) {
+        const int c = tid + i * Tile::NT;
+        const int row = c / (KP / 8), col = (c % (KP / 8)) * 8;
+        kreg[i] = (c < Tile::K_CHUNKS) ? gather(Kb, n0 + row, col, p.N, p.K) : u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int i = 0; i < Tile::V_IT; ++i) {
+        const int c = tid + i * Tile::NT;
+        const int row = c / (OP / 8), col = (c % (OP / 8)) * 8;
+        vreg[i] = (c < Tile::V_CHUNKS) ? gather(Vb, n0 + row, col, p.N, p.O) : u32x4{0, 0, 0, 0};
+      }
+    };
+    auto store_tiles = [&](int stage) {
+      T* dK = sK + stage * BN * KPI;
+      T* dV = sV + stage * BN * VPI;
+#pragma unroll
+      for (int i = 0; i < Tile::K_IT; ++i) {
+        const int c = tid + i * Tile::NT;
+        const int row = c / (KP / 8), col = (c % (KP / 8)) * 8;
+        if (c < Tile::K_CHUNKS) *reinterpret_cast<u32x4*>(dK + row * KPI + col) = kreg[i];
+      }
+#pragma unroll
+      for (int i = 0; i < Tile::V_IT; ++i) {
+        const int c = tid + i * Tile::NT;
+        const int row = c / (OP / 8), col = (c % (OP / 8)) * 8;
+        if (c < Tile::V_CHUNKS) *reinterpret_cast<u32x4*>(dV + row * VPI + col) = vreg[i];
+      }
+    };
+
+    // keys this workgroup has to visit (causal: nothing right of the last query row)
+    int n_end = p.N;
+    if (p.causal) {
+      const int last = m0 + Tile::BM;
+      n_end = last < n_end ? last : n_end;
+    }
+    const int n_tiles = (n_end + BN - 1) / BN;
+
+    f32x16 oacc[OT];
+#pragma unroll
+    for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[ot][e] = 0.0f;
+    float m_run = -INFINITY;  // running max of the scaled scores of this lane's row (log2 domain)
+    float l_run = 0.0f;       // running sum over this lane's half of the keys
+
+    if (n_tiles > 0) {
+      load_tiles(0);
+      store_tiles(0);
+    }
+    __syncthreads();
+
+    // source-lane address pattern of the LDS transpose read (see file header):
+    // 16-lane block = one 4-key x 16-column patch; lane i of the block points at
+    // key i/4, columns 4*(i%4)..+3 of the patch.
+    const int tr_i = lane & 15;
+    const int tr_row = tr_i >> 2;
+    const int tr_col = ((lane >> 4) & 1) * 16 + (tr_i & 3) * 4;
+
+    for (int t = 0; t < n_tiles; ++t) {
+      const int cur = t & 1;
+      const bool has_next = (t + 1) < n_tiles;
+      if (has_next) load_tiles((t + 1) * BN);
+      const T* cK = sK + cur * BN * KPI;
+      const T* cV = sV + cur * BN * VPI;
+
+#pragma unroll
+      for (int blk = 0; blk < BN / 32; ++blk) {
+        const int nb = t * BN + blk * 32;  // first key of this 32-key block
+        // ---- S^T block: rows = keys, columns = this wave's 32 query rows
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const vec8 kf = *reinterpret_cast<const vec8*>(cK + (blk * 32 + r32) * KPI + ks * 16 + h * 8);
+          s = Tr::mfma32(kf, qf[ks], s);
+        }
+        // lane holds keys nb + 8 g + 4 h + r (element 4 g + r) of query row q_row
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int n = nb + (e >> 2) * 8 + h * 4 + (e & 3);
+          float v = s[e] * p.scale_log2e;
+          const bool masked = (n >= p.N) || (p.causal && n > q_row);
+          v = masked ? -INFINITY : v;
+          s[e] = v;
+          tmax = fmaxf(tmax, v);
+        }
+        tmax = max_across_halves(tmax);
+        const float m_new = fmaxf(m_run, tmax);
+        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // fully masked so far
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);  // 0 when m_run = -inf
+        float psum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float pe = __builtin_amdgcn_exp2f(s[e] - m_safe);
+          s[e] = pe;
+          psum += pe;
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+          for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[ot][e] *= alpha;
+        }
+        // ---- O^T += V^T P^T over the block's two 16-key steps
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          vec8 pf;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pf[j] = Tr::from_float(s[st * 8 + j]);
+#pragma unroll
+          for (int ot = 0; ot < OT; ++ot) {
+            const T* vb = cV + (blk * 32 + st * 16 + h * 4 + tr_row) * VPI + ot * 32 + tr_col;
+            const vec4 lo = AttnVec<T>::tr_read(vb);
+            const vec4 hi = AttnVec<T>::tr_read(vb + 8 * VPI);
+            vec8 vf;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              vf[j] = lo[j];
+              vf[4 + j] = hi[j];
+            }
+            oacc[ot] = Tr::mfma32(vf, pf, oacc[ot]);
+          }
+        }
+      }
+
+      if (has_next) store_tiles(cur ^ 1);
+      __syncthreads();
+    }
+
+    // ---- normalise and store permuted: out[b / G][m][b % G][o]
+    const float l_tot = sum_across_halves(l_run);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (q_row < p.M) {
+      T* orow = reinterpret_cast<T*>(p.out) + (((int64_t)(b / p.G) * p.M + q_row) * p.G + (b % p.G)) * p.O;
+      const bool vec_ok = ((p.O & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 7) == 0);
+#pragma unroll
+      for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int o = ot * 32 + g * 8 + h * 4;
+          if (o >= p.O) continue;
+          if (vec_ok) {
+            vec4 ov;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ov[j] = Tr::from_float(oacc[ot][g * 4 + j] * inv);
+            *reinterpret_cast<vec4*>(orow + o) = ov;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (o + j < p.O) orow[o + j] = Tr::from_float(oacc[ot][g * 4 + j] * inv);
+          }
+        }
+    }
+    __syncthreads();  // LDS stage 0 is refilled by the next batch iteration
+  }
+}
+
+}  // namespace aitamd

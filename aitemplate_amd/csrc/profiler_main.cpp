@@ -218,6 +218,54 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
   return printed > 0 ? 0 : 3;
 }
 
+int profile_attention(int dtype, int64_t B, int64_t M, int64_t N, int64_t K, int64_t O, int64_t G, int causal) {
+  const size_t set_bytes = 2 * (size_t)(B * (M * K + N * K + N * O + M * O));
+  int sets = (int)(kPoolTargetBytes / (set_bytes ? set_bytes : 1)) + 1;
+  if (sets > kMaxSets) sets = kMaxSets;
+  std::vector<OperandSet> pool(sets);
+  for (int s = 0; s < sets; ++s) {
+    OperandSet& o = pool[s];
+    if (s == 0) {
+      o.a = alloc_random((size_t)(B * M * K), dtype, 1.7320508f, 21);
+      o.b = alloc_random((size_t)(B * N * K), dtype, 1.7320508f, 22);
+      o.d0 = alloc_random((size_t)(B * N * O), dtype, 1.7320508f, 23);
+    } else {
+      o.a = alloc_copy_of(pool[0].a);
+      o.b = alloc_copy_of(pool[0].b);
+      o.d0 = alloc_copy_of(pool[0].d0);
+    }
+    o.c.bytes = (size_t)(B * M * O) * 2;
+    if (o.c.bytes) HIP_OK(hipMalloc(&o.c.p, o.c.bytes));
+  }
+  const int warmup = env_int("AITAMD_PROF_WARMUP", 3);
+  const int iters = env_int("AITAMD_PROF_ITERS", 10);
+  const float scale = K > 0 ? 1.0f / sqrtf((float)K) : 1.0f;
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  hipEvent_t e0, e1;
+  HIP_OK(hipEventCreate(&e0));
+  HIP_OK(hipEventCreate(&e1));
+  auto launch = [&](const OperandSet& o) {
+    return aitamd_bmm_softmax_bmm_permute(dtype, o.a.p, o.b.p, o.d0.p, o.c.p, B, M, N, K, O, G, scale, causal, stream);
+  };
+  for (int i = 0; i < warmup; ++i) {
+    if (launch(pool[i % sets]) != 0) {
+      fprintf(stderr, "attention launch failed: %s\n", aitamd_last_error());
+      return 3;
+    }
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipEventRecord(e0, stream));
+  for (int i = 0; i < iters; ++i) launch(pool[i % sets]);
+  HIP_OK(hipEventRecord(e1, stream));
+  HIP_OK(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  printf("OP:attention_f%s_q128_kv64,TIME:%.6f,WS:0\n", dtype == 0 ? "16" : "b16", ms / (iters > 0 ? iters : 1));
+  HIP_OK(hipStreamDestroy(stream));
+  return 0;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -237,6 +285,10 @@ int main(int argc, char** argv) {
   if (kind == "bmm") {
     if (d.size() < 4) return 2;
     return profile_gemm_like(op, dtype, d[0], d[1], d[2], d[3], true);
+  }
+  if (kind == "attn") {
+    if (d.size() < 6) return 2;
+    return profile_attention(dtype, d[0], d[1], d[2], d[3], d[4], d[5], d.size() > 6 ? (int)d[6] : 0);
   }
   fprintf(stderr, "unknown kind %s\n", kind.c_str());
   return 2;

@@ -115,3 +115,29 @@ def bmm_rcr(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None
                             M * N, _stream_ptr())
     _kernels.check(rc, "bmm_rcr")
     return out
+
+
+def bmm_softmax_bmm_permute(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, shape, scale: float = 1.0,
+                            causal: bool = False, layout: str = "0213",
+                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """softmax(scale * q @ k^T) @ v with the [B, M, O] result written as [B / G, M, G, O], G = shape[0]
+    (python/aitemplate/compiler/ops/gemm_universal/bmm_softmax_bmm_permute.py:30-194)."""
+    lib = _kernels.load()
+    if layout != "0213":
+        raise NotImplementedError(f"{layout} is not implemented!")
+    dtype = q.dtype
+    for t, n in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
+        _check(t, n, dtype)
+    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+        raise ValueError("bmm_softmax_bmm_permute operands must be contiguous")
+    B, M, K = q.shape
+    N, O = v.shape[1], v.shape[2]
+    if k.shape != (B, N, K) or v.shape[0] != B:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    G = int(shape[0])
+    if out is None:
+        out = torch.empty(B // G, M, G, O, dtype=dtype, device=q.device)
+    rc = lib.aitamd_bmm_softmax_bmm_permute(_TORCH_DTYPE_ID[dtype], _p(q), _p(k), _p(v), _p(out), B, M, N, K, O, G,
+                                            float(scale), int(bool(causal)), _stream_ptr())
+    _kernels.check(rc, "bmm_softmax_bmm_permute")
+    return out

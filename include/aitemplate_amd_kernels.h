@@ -121,6 +121,20 @@ AITAMD_API int aitamd_bmm_rcr(int dtype, int algo,
                               int64_t stride_a, int64_t stride_b, int64_t stride_c,
                               void* stream);
 
+/* out[b / G, m, b % G, o] = sum_n softmax_n( scale * sum_k Q[b,m,k] K[b,n,k] ) V[b,n,o]
+ * Q [B,M,K], K [B,N,K], V [B,N,O] contiguous; out [B/G, M, G, O] (the "0213"
+ * permute of [B/G, G, M, O]); G = number of heads, B % G == 0.  `scale` is
+ * rounded to the element type first, as the reference does; causal != 0 masks
+ * keys n > m.  K and O up to 128; head dims that are not MFMA multiples are
+ * padded on chip only.  Rows whose keys are all masked (N == 0) produce 0.
+ * Replaces the generated bmm_softmax_bmm_permute op function's CK call
+ * (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:84-110,
+ * frontend python/aitemplate/compiler/ops/gemm_universal/bmm_softmax_bmm_permute.py:30-194). */
+AITAMD_API int aitamd_bmm_softmax_bmm_permute(int dtype,
+                                              const void* q, const void* k, const void* v, void* out,
+                                              int64_t B, int64_t M, int64_t N, int64_t K, int64_t O,
+                                              int64_t G, float scale, int causal, void* stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

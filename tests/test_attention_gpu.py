@@ -1,0 +1,100 @@
+"""GPU parity of bmm_softmax_bmm_permute through the C ABI against the CPU oracle.
+Tolerance atol = rtol = 2e-2 (softmax path, fp16 out / fp32 accumulate)."""
+import pytest
+import torch
+
+from aitemplate_amd import eager
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-2
+
+
+def _rand(shape, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g).to(dtype)
+
+
+def _check(B, M, N, K, O, G, causal=False, dtype=torch.float16, scale=None, seed=0, tol=TOL):
+    print(f"case attention B={B} M={M} N={N} K={K} O={O} G={G} causal={causal} {dtype}", flush=True)
+    q, k, v = _rand((B, M, K), dtype, seed), _rand((B, N, K), dtype, seed + 1), _rand((B, N, O), dtype, seed + 2)
+    scale = K ** -0.5 if scale is None else scale
+    want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, scale, G, causal).to(dtype).float()
+    got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=scale, causal=causal)
+    torch.cuda.synchronize()
+    assert got.shape == (B // G, M, G, O)
+    torch.testing.assert_close(got.cpu().float(), want, atol=tol, rtol=tol)
+
+
+# the shapes of the reference's ROCm test (tests/unittest/ops/test_bmm_softmax_bmm.py:174-205)
+@pytest.mark.parametrize("B,M,N,K,O,G,causal", [
+    (24, 256, 256, 64, 64, 12, False),
+    (24, 196, 196, 64, 64, 12, False),
+    (24, 128, 1024, 64, 128, 12, False),
+    (24, 128, 49, 64, 128, 12, False),
+    (24, 49, 49, 64, 64, 12, False),
+    (24, 1020, 1020, 64, 128, 12, False),
+    (32, 49, 49, 64, 64, 4, False),
+    (16, 4096, 64, 40, 40, 8, False),
+    (12, 64, 64, 64, 64, 12, True),
+])
+def test_reference_shapes(B, M, N, K, O, G, causal):
+    _check(B, M, N, K, O, G, causal)
+
+
+@pytest.mark.parametrize("B,M,N,K,O,G,causal", [
+    (4, 130, 70, 40, 40, 2, False),     # ragged M and N, head_dim 40
+    (2, 33, 200, 16, 24, 1, False),     # small head dims
+    (2, 65, 65, 128, 128, 2, True),     # largest head dims, causal with ragged edge
+    (4, 300, 300, 96, 80, 4, True),
+    (2, 17, 9, 20, 12, 2, False),       # K, O not multiples of 8 -> element-wise loads
+    (3, 5, 1, 8, 8, 3, False),          # a single key: softmax == 1
+])
+def test_ragged_and_odd_shapes(B, M, N, K, O, G, causal):
+    _check(B, M, N, K, O, G, causal, seed=3)
+
+
+def test_bf16():
+    _check(8, 200, 136, 64, 64, 4, dtype=torch.bfloat16, tol=4e-2)
+    _check(8, 100, 100, 40, 40, 8, causal=True, dtype=torch.bfloat16, tol=4e-2)
+
+
+def test_large_scores_do_not_overflow():
+    # scores of magnitude ~60: exp() of the raw score would overflow fp16/fp32 ranges without the running max
+    _check(4, 64, 256, 64, 64, 4, scale=1.0, seed=5, tol=3e-2)
+
+
+def test_invariants_on_gpu():
+    B, M, N, K, O, G = 8, 100, 150, 40, 40, 4
+    q, k = _rand((B, M, K), torch.float16, 1).cuda(), _rand((B, N, K), torch.float16, 2).cuda()
+    vc = torch.full((B, N, O), 0.75, dtype=torch.float16, device="cuda")
+    out = eager.bmm_softmax_bmm_permute(q, k, vc, (G,), scale=0.2)
+    assert torch.allclose(out.float().cpu(), torch.full((B // G, M, G, O), 0.75), atol=2e-3)
+    vb = torch.arange(B, dtype=torch.float32).reshape(B, 1, 1).expand(B, N, O).to(torch.float16).cuda().contiguous()
+    out = eager.bmm_softmax_bmm_permute(q, k, vb, (G,), scale=0.2).cpu().float()
+    for b in range(B):
+        assert torch.allclose(out[b // G, :, b % G, :], torch.full((M, O), float(b)), atol=1e-2)
+
+
+def test_empty_keys_give_zero_and_empty_batch_is_noop():
+    q = torch.randn(2, 8, 16, dtype=torch.float16, device="cuda")
+    k = torch.empty(2, 0, 16, dtype=torch.float16, device="cuda")
+    v = torch.empty(2, 0, 8, dtype=torch.float16, device="cuda")
+    out = torch.full((1, 8, 2, 8), 7.0, dtype=torch.float16, device="cuda")
+    eager.bmm_softmax_bmm_permute(q, k, v, (2,), out=out)
+    torch.cuda.synchronize()
+    assert float(out.abs().max()) == 0.0
+    with pytest.raises(RuntimeError):
+        eager.bmm_softmax_bmm_permute(q, k, v, (3,))  # batch 2 is not a multiple of 3 heads
+
+
+def test_config_c5_full_size():
+    print("case config=c5 full size", flush=True)
+    inp = oracle.config_inputs("c5")
+    want = oracle.config_expected("c5", inp).half().float()
+    got = eager.bmm_softmax_bmm_permute(inp["q"].cuda(), inp["k"].cuda(), inp["v"].cuda(), (oracle.C5_HEADS,),
+                                        scale=oracle.C5_SCALE)
+    torch.cuda.synchronize()
+    assert got.shape == (2, 4096, 8, 40)
+    torch.testing.assert_close(got.cpu().float(), want, atol=TOL, rtol=TOL)
