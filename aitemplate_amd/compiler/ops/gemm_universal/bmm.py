@@ -1,0 +1,74 @@
+"""Batched GEMM: the bmm base class and bmm_rcr.
+
+Counterparts: python/aitemplate/compiler/ops/gemm_universal/bmm.py:69-119 (base, batch
+broadcast rules) and bmm_xxx.py:22-150,261-278 (layout bookkeeping; only the r-c-r
+layout exists on this backend)."""
+from ...base import Tensor
+from ...dtype import is_same_dtype
+from . import gemm_common as common
+
+
+class bmm(common.gemm):
+    """Base class for bmm: operands are 3-D, or 2-D and broadcast over the other's batch."""
+
+    def _get_batch_size(self, a: Tensor, b: Tensor):
+        self._sanity_check(a, b)
+        a_shapes, b_shapes = a._attrs["shape"], b._attrs["shape"]
+        if len(a_shapes) == 2:
+            return b_shapes[0]
+        if len(b_shapes) == 2:
+            return a_shapes[0]
+        if a_shapes[0] != b_shapes[0] and a_shapes[0] != 1 and b_shapes[0] != 1:
+            raise RuntimeError(
+                "bmm operand A and B should have same batch_size, or batch_size = 1! "
+                f"Current shape A: {a_shapes} shape B: {b_shapes} .")
+        return a_shapes[0] if a_shapes[0] != 1 else b_shapes[0]
+
+    def _sanity_check(self, a: Tensor, b: Tensor):
+        a_shapes, b_shapes = a._attrs["shape"], b._attrs["shape"]
+        if len(a_shapes) not in (2, 3):
+            raise RuntimeError(f"bmm operand A should have 2 or 3 dimensions! Current shape: {a_shapes}.")
+        if len(b_shapes) not in (2, 3):
+            raise RuntimeError(f"bmm operand B should have 2 or 3 dimensions! Current shape: {b_shapes}.")
+        if len(a_shapes) == 2 and len(b_shapes) == 2:
+            raise RuntimeError("bmm operand A and B both have 2 dimensions! Use gemm instead.")
+        if not is_same_dtype(a.dtype(), b.dtype()):
+            raise RuntimeError(
+                f"gemm operand A and B should have the same data type! Current A: {a.dtype()}, B: {b.dtype()}.")
+
+
+class bmm_rcr(bmm):
+    """C[b] = A[b] @ B[b]^T with A [B, M, K], B [B, N, K] -> C [B, M, N]
+    (torch.bmm(A, B.transpose(2, 1)))."""
+
+    def __init__(self):
+        super().__init__()
+        self._attrs["op"] = "bmm_rcr"
+
+        def cal_align_ab(m, n, k):
+            return common.default_align_ab(k, k, self._attrs["inputs"][0].dtype())
+
+        self._attrs["f_ab_alignment"] = cal_align_ab
+
+    def _infer_shapes(self, a: Tensor, b: Tensor):
+        a_shape, b_shape = a.shape(), b.shape()
+        if a_shape[-1] != b_shape[-1]:
+            raise RuntimeError(f"bmm_rcr operand A and B should have the same K dim! A: {a_shape}, B: {b_shape}")
+        return [self._get_batch_size(a, b), a_shape[-2], b_shape[-2]]
+
+    def _extract_dims(self, for_profiling: bool = False):
+        a_shapes = common.extract_shape_from_accessor(self._attrs, common.Source.INPUT, 0)
+        b_shapes = common.extract_shape_from_accessor(self._attrs, common.Source.INPUT, 1)
+        out_shapes = common.extract_shape_from_accessor(self._attrs, common.Source.OUTPUT, 0)
+        b_dim = common.create_input_batch_diminfo([a_shapes, b_shapes], [0, 0], out_shapes[0])
+        b_dim.append(common.DimInfo(common.Source.OUTPUT, tensor_idx=0, dim_idx=0))
+        ra, rb = len(a_shapes), len(b_shapes)
+        return {
+            "B": b_dim,
+            "M": [common.DimInfo(common.Source.INPUT, tensor_idx=0, dim_idx=ra - 2),
+                  common.DimInfo(common.Source.OUTPUT, tensor_idx=0, dim_idx=1)],
+            "N": [common.DimInfo(common.Source.INPUT, tensor_idx=1, dim_idx=rb - 2),
+                  common.DimInfo(common.Source.OUTPUT, tensor_idx=0, dim_idx=2)],
+            "K": [common.DimInfo(common.Source.INPUT, tensor_idx=0, dim_idx=ra - 1),
+                  common.DimInfo(common.Source.INPUT, tensor_idx=1, dim_idx=rb - 1)],
+        }

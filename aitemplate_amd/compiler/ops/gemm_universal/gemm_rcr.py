@@ -1,0 +1,41 @@
+"""gemm_rcr: A[M.., K] row-major  x  B[N, K] ("column-major" B, i.e. K-contiguous rows)  ->  C[M.., N].
+
+Equivalent to torch.nn.functional.linear(A, B).
+Counterpart of python/aitemplate/compiler/ops/gemm_universal/gemm_rcr.py:26-112."""
+from ...base import IntImm, Tensor
+from . import gemm_common as common
+
+
+class gemm_rcr(common.gemm):
+    def __init__(self):
+        super().__init__()
+        self._attrs["op"] = "gemm_rcr"
+
+        def cal_align_ab(m, n, k):
+            return common.default_align_ab(k, k, self._attrs["inputs"][0].dtype())
+
+        self._attrs["f_ab_alignment"] = cal_align_ab
+
+    def _infer_shapes(self, a: Tensor, b: Tensor):
+        return a._attrs["shape"][:-1] + [b._attrs["shape"][0]]
+
+    def _extract_dims(self, for_profiling: bool = False):
+        # leading dims of A are folded into M
+        a_rank = 2 if for_profiling else len(self._attrs["input_accessors"][0].original_shapes)
+        lead = list(range(a_rank - 1))
+        return {
+            "M": [common.DimInfo(common.Source.INPUT, tensor_idx=0, dim_idx=lead),
+                  common.DimInfo(common.Source.OUTPUT, tensor_idx=0, dim_idx=lead)],
+            "N": [common.DimInfo(common.Source.INPUT, tensor_idx=1, dim_idx=0),
+                  common.DimInfo(common.Source.OUTPUT, tensor_idx=0, dim_idx=a_rank - 1)],
+            "K": [common.DimInfo(common.Source.INPUT, tensor_idx=0, dim_idx=a_rank - 1),
+                  common.DimInfo(common.Source.INPUT, tensor_idx=1, dim_idx=1)],
+        }
+
+    def _align_ab(self, a: Tensor, b: Tensor):
+        a_shape, b_shape = a._attrs["shape"], b._attrs["shape"]
+        if a_shape[-1] != b_shape[-1]:
+            raise RuntimeError(f"A/B shape mismatch! A: {a_shape}, B: {b_shape}")
+        if not isinstance(a_shape[-1], IntImm):
+            raise RuntimeError(f"K must be static! k: {a_shape[-1]}")
+        return a, b

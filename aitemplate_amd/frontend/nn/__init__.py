@@ -1,0 +1,3 @@
+from .linear import Linear  # noqa: F401
+from .module import Module  # noqa: F401
+from .parameter import Parameter  # noqa: F401

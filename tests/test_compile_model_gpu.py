@@ -1,0 +1,197 @@
+"""End-to-end parity through the unchanged boundary: graph -> compile_model() -> test.so ->
+AITemplateModelContainerRun, written the way the reference's own ROCm unit tests are
+(tests/unittest/ops/test_gemm.py, test_gemm_bias.py, test_gemm_bias_relu.py,
+test_gemm_rcr_bias_fast_gelu.py, test_gemm_bias_broadcast.py, test_bmm.py,
+test_bmm_softmax_bmm.py) but checked against the CPU oracle at atol = rtol = 1e-2
+(2e-2 on the softmax path)."""
+import itertools
+import os
+
+import pytest
+import torch
+
+from aitemplate_amd.compiler import compile_model, ops
+from aitemplate_amd.frontend import IntImm, Tensor
+from aitemplate_amd.testing import detect_target
+from aitemplate_amd.utils import shape_utils
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+WORKDIR = os.environ.get("AIT_TEST_WORKDIR", "/tmp/aitemplate_amd_tests")
+_counter = itertools.count()
+
+
+def _rand(shape, seed, scale=1.0, dtype=torch.float16):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def _mark_output(y, name="output_0"):
+    y._attrs["name"] = name
+    y._attrs["is_output"] = True
+    return y
+
+
+def _build_gemm(op_name, Ms, N, K, dtype="float16"):
+    m_dim = shape_utils.gen_int_var_min_max(Ms, name="m")
+    X = Tensor(shape=[m_dim, IntImm(K)], dtype=dtype, name="input_0", is_input=True)
+    W = Tensor(shape=[IntImm(N), IntImm(K)], dtype=dtype, name="input_1", is_input=True)
+    inputs = [X, W]
+    if op_name != "gemm_rcr":
+        inputs.append(Tensor(shape=[IntImm(N)], dtype=dtype, name="input_2", is_input=True))
+    nres = {"gemm_rcr_bias_add": 1, "gemm_rcr_bias_add_add": 2, "gemm_rcr_bias_add_relu": 1,
+            "gemm_rcr_bias_mul_add": 2}.get(op_name, 0)
+    for i in range(nres):
+        inputs.append(Tensor(shape=[m_dim, IntImm(N)], dtype=dtype, name=f"input_{3 + i}", is_input=True))
+    Y = _mark_output(getattr(ops, op_name)()(*inputs))
+    return compile_model(Y, detect_target(), WORKDIR, f"{op_name}_{next(_counter)}"), nres
+
+
+def _run_gemm_case(op_name, Ms, N, K, dtype="float16", tol=1e-2):
+    print(f"case compile_model {op_name} Ms={Ms} N={N} K={K} {dtype}", flush=True)
+    module, nres = _build_gemm(op_name, Ms, N, K, dtype)
+    tdt = {"float16": torch.float16, "bfloat16": torch.bfloat16}[dtype]
+    for M in Ms:
+        x, w, b = _rand((M, K), 1, dtype=tdt), _rand((N, K), 2, max(K, 1) ** -0.5, tdt), _rand((N,), 3, dtype=tdt)
+        ds = [_rand((M, N), 4 + i, dtype=tdt) for i in range(nres)]
+        want = oracle.torch_gemm(op_name, x, w, b, *(ds + [None] * (2 - nres))).to(tdt).float()
+        ins = {"input_0": x.cuda(), "input_1": w.cuda()}
+        if op_name != "gemm_rcr":
+            ins["input_2"] = b.cuda()
+        for i, d in enumerate(ds):
+            ins[f"input_{3 + i}"] = d.cuda()
+        y = torch.empty(M, N, dtype=tdt, device="cuda")
+        out = module.run_with_tensors(ins, [y])
+        assert tuple(out["output_0"].shape) == (M, N)
+        if M * N * K != 0:
+            torch.testing.assert_close(y.cpu().float(), want, atol=tol, rtol=tol)
+    module.close()
+
+
+def test_gemm_rcr_simple_static():          # test_gemm.py:83-84
+    _run_gemm_case("gemm_rcr", [1024], 512, 256)
+
+
+@pytest.mark.parametrize("Ms,N,K", [([4096], 4, 4), ([1000], 81, 1024), ([67200], 3, 256)])
+def test_gemm_rcr_bias_static(Ms, N, K):    # test_gemm_bias.py:96-99
+    _run_gemm_case("gemm_rcr_bias", Ms, N, K)
+
+
+def test_gemm_rcr_bias_dynamic_m():         # test_gemm_bias.py dynamic_m case
+    _run_gemm_case("gemm_rcr_bias", [1, 7, 64, 127], 64, 1024)
+
+
+def test_gemm_rcr_bias_zero_size():         # test_gemm_bias.py:81-89
+    _run_gemm_case("gemm_rcr_bias", [2], 64, 0)
+    _run_gemm_case("gemm_rcr_bias", [2], 0, 4)
+    _run_gemm_case("gemm_rcr_bias", [0], 4, 4)
+
+
+def test_gemm_rcr_bias_relu():              # test_gemm_bias_relu.py:75-76
+    _run_gemm_case("gemm_rcr_bias_relu", [128], 64, 1024)
+
+
+def test_gemm_rcr_bias_fast_gelu_and_gelu():  # test_gemm_rcr_bias_fast_gelu.py:130-136
+    _run_gemm_case("gemm_rcr_bias_fast_gelu", [128], 64, 1024)
+    _run_gemm_case("gemm_rcr_bias_gelu", [128], 64, 1024)
+
+
+def test_gemm_rcr_bias_add_and_add_add():   # test_gemm_bias_broadcast.py:193-227,350-387
+    _run_gemm_case("gemm_rcr_bias_add", [8], 8, 8)
+    _run_gemm_case("gemm_rcr_bias_add_add", [8], 8, 8)
+    _run_gemm_case("gemm_rcr_bias_add_add", [2, 300], 264, 520)
+    _run_gemm_case("gemm_rcr_bias_add_relu", [77], 72, 40)
+    _run_gemm_case("gemm_rcr_bias_mul_add", [77], 72, 40)
+
+
+def test_gemm_rcr_bias_bf16():
+    _run_gemm_case("gemm_rcr_bias", [128], 64, 1024, dtype="bfloat16", tol=3e-2)
+
+
+def test_gemm_3d_input_is_flattened():
+    X = Tensor(shape=[IntImm(4), IntImm(50), IntImm(64)], name="input_0", is_input=True)
+    W = Tensor(shape=[72, 64], name="input_1", is_input=True)
+    B = Tensor(shape=[72], name="input_2", is_input=True)
+    Y = _mark_output(ops.gemm_rcr_bias()(X, W, B))
+    module = compile_model(Y, detect_target(), WORKDIR, f"gemm_3d_{next(_counter)}")
+    x, w, b = _rand((4, 50, 64), 1), _rand((72, 64), 2, 0.125), _rand((72,), 3)
+    y = torch.empty(4, 50, 72, dtype=torch.float16, device="cuda")
+    module.run_with_tensors([x.cuda(), w.cuda(), b.cuda()], [y])
+    want = oracle.torch_gemm("gemm_rcr_bias", x.reshape(-1, 64), w, b).reshape(4, 50, 72)
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("B,M,N,K", [(1024, 128, 512, 256), (5, 33, 17, 24)])
+def test_bmm_rcr(B, M, N, K):               # test_bmm.py:69-70
+    X = Tensor(shape=[B, M, K], name="input_0", is_input=True)
+    W = Tensor(shape=[B, N, K], name="input_1", is_input=True)
+    Y = _mark_output(ops.bmm_rcr()(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"bmm_rcr_{next(_counter)}")
+    q, k = _rand((B, M, K), 1), _rand((B, N, K), 2, K ** -0.5)
+    y = torch.empty(B, M, N, dtype=torch.float16, device="cuda")
+    module.run_with_tensors([q.cuda(), k.cuda()], [y])
+    torch.testing.assert_close(y.cpu().float(), oracle.torch_bmm_rcr(q, k).half().float(), atol=1e-2, rtol=1e-2)
+
+
+def test_bmm_rcr_broadcast_2d_operand():
+    X = Tensor(shape=[6, 40, 32], name="input_0", is_input=True)
+    W = Tensor(shape=[24, 32], name="input_1", is_input=True)
+    Y = _mark_output(ops.bmm_rcr()(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"bmm_rcr_bc_{next(_counter)}")
+    q, k = _rand((6, 40, 32), 1), _rand((24, 32), 2, 0.2)
+    y = torch.empty(6, 40, 24, dtype=torch.float16, device="cuda")
+    module.run_with_tensors([q.cuda(), k.cuda()], [y])
+    torch.testing.assert_close(y.cpu().float(), oracle.torch_bmm_rcr(q, k).half().float(), atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("bs,ms,N,K,D,heads,causal,copy_op", [
+    ([24], [256], 256, 64, 64, 12, False, False),
+    ([24], [128], 49, 64, 128, 12, False, False),
+    ([24], [1020], 1020, 64, 128, 12, False, True),
+    ([16], [4096], 64, 40, 40, 8, False, False),
+    ([12], [64], 64, 64, 64, 12, True, True),
+])
+def test_bmm_softmax_bmm_permute(bs, ms, N, K, D, heads, causal, copy_op):   # test_bmm_softmax_bmm.py:174-205
+    batch_dim = shape_utils.gen_int_var_min_max(bs, name="batch_size")
+    m_dim = shape_utils.gen_int_var_min_max(ms, name="m")
+    X = Tensor(shape=[batch_dim, m_dim, K], name="input_0", is_input=True)
+    B0 = Tensor(shape=[batch_dim, N, K], name="input_1", is_input=True)
+    B1 = Tensor(shape=[batch_dim, N, D], name="input_2", is_input=True)
+    scale = 64 ** -0.5
+    OP = ops.bmm_softmax_bmm_permute(shape=(heads,), scale=scale, causal=causal)
+    if copy_op:
+        OP = ops.bmm_softmax_bmm_permute(**OP._get_op_attributes())
+    Y = _mark_output(OP(X, B0, B1))
+    module = compile_model(Y, detect_target(), WORKDIR, f"attn_{next(_counter)}", dll_name=f"test_{next(_counter)}.so")
+    for b, m in itertools.product(bs, ms):
+        q, k, v = _rand((b, m, K), 1), _rand((b, N, K), 2), _rand((b, N, D), 3)
+        want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, scale, heads, causal).half().float()
+        y = torch.empty(b // heads, m, heads, D, dtype=torch.float16, device="cuda")
+        module.run_with_tensors([q.cuda(), k.cuda(), v.cuda()], [y])
+        torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
+
+
+# ---- the five benchmark configurations, full size, through the C ABI ----------------------
+@pytest.mark.parametrize("cfg", ["c1", "c2a", "c2b", "c3", "c4", "c5"])
+def test_benchmark_config_through_compile_model(cfg):
+    print(f"case compile_model config={cfg}", flush=True)
+    inp = oracle.config_inputs(cfg)
+    op_name = oracle.CONFIG_OP[cfg]
+    order = [k for k in ("x", "w", "bias", "d0", "d1", "q", "k", "v") if k in inp]
+    tensors = [Tensor(shape=list(inp[k].shape), name=f"input_{i}", is_input=True) for i, k in enumerate(order)]
+    if cfg == "c5":
+        Y = ops.bmm_softmax_bmm_permute(shape=(oracle.C5_HEADS,), scale=oracle.C5_SCALE)(*tensors)
+        tol = 2e-2
+    else:
+        Y = getattr(ops, op_name)()(*tensors)
+        tol = 1e-2
+    _mark_output(Y)
+    module = compile_model(Y, detect_target(), WORKDIR, f"config_{cfg}")
+    want = oracle.config_expected(cfg, inp).half().float()
+    y = torch.empty(*want.shape, dtype=torch.float16, device="cuda")
+    module.run_with_tensors([inp[k].cuda() for k in order], [y])
+    torch.testing.assert_close(y.cpu().float(), want, atol=tol, rtol=tol)
+    # timing through the ABI works and is positive
+    mean, std, _ = module.benchmark_with_tensors([inp[k].cuda() for k in order], [y], count=5, repeat=2)
+    assert mean > 0
