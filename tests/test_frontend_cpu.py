@@ -1,0 +1,342 @@
+"""Host-side logic, no GPU: op construction and shape inference, exec keys and profiler command
+lines (golden strings from the reference's formats), registry, naming, memory planning, code
+generation, the model build and the exported C ABI, and the profiler runner with fake commands
+(the latter mirrors tests/unittest/backend/test_profiler.py:48-66)."""
+import copy
+import ctypes
+import os
+import re
+import stat
+import subprocess
+import sys
+from random import random
+from time import sleep
+
+import pytest
+
+from aitemplate_amd.backend import registry
+from aitemplate_amd.backend.profiler_runner import ProfilerRunner, extract_profile_result
+from aitemplate_amd.compiler import compile_model, ops, transform
+from aitemplate_amd.compiler.base import DynamicProfileStrategy, IntImm, IntVar, Tensor
+from aitemplate_amd.compiler.ops.gemm_universal.gemm_common import gemm_inverse_key_func
+from aitemplate_amd.compiler.transform.name_graph import reset_name_counters
+from aitemplate_amd.frontend import nn
+from aitemplate_amd.testing import detect_target
+from aitemplate_amd.utils import alignment, shape_utils
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _gemm_bias_graph(Ms=(256,), N=1024, K=1024, op="gemm_rcr_bias"):
+    m = shape_utils.gen_int_var_min_max(list(Ms), name="m")
+    X = Tensor(shape=[m, IntImm(K)], name="input_0", is_input=True)
+    W = Tensor(shape=[IntImm(N), IntImm(K)], name="input_1", is_input=True)
+    B = Tensor(shape=[IntImm(N)], name="input_2", is_input=True)
+    Y = getattr(ops, op)()(X, W, B)
+    Y._attrs["name"] = "output_0"
+    Y._attrs["is_output"] = True
+    return Y
+
+
+# ---- IR -------------------------------------------------------------------------------
+def test_intvar_intimm_semantics():
+    assert IntImm(4) == 4 and IntImm(4) == IntImm(4) and IntImm(4) != IntImm(5)
+    with pytest.raises(RuntimeError):
+        IntImm(1.5)
+    with pytest.raises(RuntimeError):
+        IntVar([3])
+    with pytest.raises(RuntimeError):
+        IntVar([-1, 4])
+    v = IntVar([8, 2, 4], name="b")
+    assert (v.lower_bound(), v.upper_bound()) == (2, 8)
+    assert IntVar([1, 9], name="b") == v  # same symbol
+    assert isinstance(shape_utils.gen_int_var_min_max([7, 7]), IntImm)
+    assert isinstance(shape_utils.gen_int_var_min_max([1, 7]), IntVar)
+    t = Tensor([3, v])
+    assert [type(d).__name__ for d in t.shape()] == ["IntImm", "IntVar"]
+    assert t.size_bytes() == 3 * 8 * 2
+    with pytest.raises(RuntimeError):
+        Tensor(["x"])
+
+
+def test_alignment_helpers():
+    assert alignment.find_max_alignment(1024, "float16") == 8
+    assert alignment.find_max_alignment(4, "float16") == 4
+    assert alignment.find_max_alignment(81, "float16") == 1
+    assert alignment.find_max_alignment(6, "float32") == 2
+
+
+# ---- ops ------------------------------------------------------------------------------
+def test_gemm_shape_inference_and_attrs():
+    Y = _gemm_bias_graph()
+    op = list(Y.src_ops())[0]
+    assert [d.value() for d in Y.shape()] == [256, 1024]
+    for key in ("op", "has_profiler", "f_ab_alignment", "epilogue_alignment", "epilogue", "workspace", "split_k",
+                "num_sources", "alpha", "permute_shape", "inputs", "input_accessors", "outputs",
+                "output_accessors"):
+        assert key in op._attrs, key
+    assert op._attrs["op"] == "gemm_rcr_bias" and op._attrs["epilogue_alignment"] == 8
+    # leading dims of A are flattened into M
+    X3 = Tensor([4, 50, 64])
+    Y3 = ops.gemm_rcr()(X3, Tensor([72, 64]))
+    assert [d.value() for d in Y3.shape()] == [4, 50, 72]
+
+
+def test_gemm_argument_errors():
+    with pytest.raises(RuntimeError, match="A/B shape mismatch"):
+        ops.gemm_rcr()(Tensor([4, 8]), Tensor([4, 16]))
+    with pytest.raises(RuntimeError, match="K must be static"):
+        kdim = IntVar([1, 8], name="k")
+        ops.gemm_rcr()(Tensor([4, kdim]), Tensor([4, kdim]))
+    with pytest.raises(RuntimeError, match="Bias should be 1D"):
+        ops.gemm_rcr_bias()(Tensor([4, 8]), Tensor([6, 8]), Tensor([1, 6]))
+    with pytest.raises(RuntimeError, match="doesn't match"):
+        ops.gemm_rcr_bias()(Tensor([4, 8]), Tensor([6, 8]), Tensor([5]))
+    with pytest.raises(RuntimeError, match="doesn't match gemm_bias"):
+        ops.gemm_rcr_bias_add()(Tensor([4, 8]), Tensor([6, 8]), Tensor([6]), Tensor([4, 5]))
+    with pytest.raises(RuntimeError):
+        ops.gemm_rcr_bias_add_add()(Tensor([4, 8]), Tensor([6, 8]), Tensor([6]), Tensor([4, 6]))  # needs d1
+    with pytest.raises(RuntimeError, match="same data type"):
+        ops.gemm_rcr()(Tensor([4, 8]), Tensor([6, 8], dtype="float32"))
+    with pytest.raises(RuntimeError, match="2 dimensions"):
+        ops.gemm_rcr()(Tensor([4, 8]), Tensor([2, 6, 8]))
+
+
+def test_exec_keys_are_the_reference_format():
+    op = list(_gemm_bias_graph().src_ops())[0]
+    op._extract_exec_path(DynamicProfileStrategy.MAX)
+    assert list(op._attrs["exec_path"]) == ["M == 256 && N == 1024 && K == 1024"]
+    assert gemm_inverse_key_func("M == 256 && N == 1024 && K == 1024") == [256, 1024, 1024]
+    op = list(_gemm_bias_graph(Ms=(1, 1024), N=64, K=32).src_ops())[0]
+    op._extract_exec_path(DynamicProfileStrategy.MAX)
+    item = list(op._attrs["exec_path"].values())[0]
+    assert item.profiling_key == "M == 1024 && N == 64 && K == 32"
+    assert item.exec_cond == "M >= 1 && M <= 1024 && N == 64 && K == 32"
+    op._extract_exec_path(DynamicProfileStrategy.MIN)
+    assert list(op._attrs["exec_path"]) == ["M == 1 && N == 64 && K == 32"]
+    with pytest.raises(NotImplementedError):
+        op._extract_exec_path(DynamicProfileStrategy.HINTS)
+    # bmm keys are ordered B, M, N, K; attention B, M, N, K, O
+    b = ops.bmm_rcr()
+    b(Tensor([768, 384, 64]), Tensor([768, 384, 64]))
+    b._extract_exec_path(DynamicProfileStrategy.MAX)
+    assert list(b._attrs["exec_path"]) == ["B == 768 && M == 384 && N == 384 && K == 64"]
+    a = ops.bmm_softmax_bmm_permute(shape=(8,), scale=0.5)
+    a(Tensor([16, 4096, 40]), Tensor([16, 4096, 40]), Tensor([16, 4096, 40]))
+    a._extract_exec_path(DynamicProfileStrategy.MAX)
+    assert list(a._attrs["exec_path"]) == ["B == 16 && M == 4096 && N == 4096 && K == 40 && O == 40"]
+
+
+def test_bmm_rules():
+    y = ops.bmm_rcr()(Tensor([6, 40, 32]), Tensor([24, 32]))
+    assert [d.value() for d in y.shape()] == [6, 40, 24]
+    y = ops.bmm_rcr()(Tensor([1, 40, 32]), Tensor([5, 24, 32]))
+    assert [d.value() for d in y.shape()] == [5, 40, 24]
+    with pytest.raises(RuntimeError, match="same batch_size"):
+        ops.bmm_rcr()(Tensor([2, 40, 32]), Tensor([3, 24, 32]))
+    with pytest.raises(RuntimeError, match="Use gemm instead"):
+        ops.bmm_rcr()(Tensor([40, 32]), Tensor([24, 32]))
+
+
+def test_attention_op_output_attrs_and_copy():
+    op = ops.bmm_softmax_bmm_permute(shape=(8,), scale=0.158, causal=True)
+    out = op(Tensor([16, 4096, 40]), Tensor([16, 4096, 40]), Tensor([16, 4096, 40]))
+    assert [d.value() for d in out.shape()] == [2, 4096, 8, 40]
+    assert out._attrs["is_view_of"] is op._attrs["outputs"][0]
+    assert op._attrs["op"] == "bmm_softmax_bmm_permute_causal"
+    attrs = op._get_op_attributes()
+    assert attrs == {"causal": True, "layout": "0213", "scale": 0.158, "shape": (8,)}
+    clone = ops.bmm_softmax_bmm_permute(**attrs)
+    assert clone._attrs["op"] == op._attrs["op"] and clone._attrs["layout"] == op._attrs["layout"]
+    dc = copy.deepcopy(op)
+    assert dc._attrs["scale"] == 0.158 and dc is not op
+    with pytest.raises(NotImplementedError):
+        ops.bmm_softmax_bmm_permute(shape=(8,), layout="0123")(Tensor([16, 8, 8]), Tensor([16, 8, 8]), Tensor([16, 8, 8]))
+
+
+def test_nn_linear_picks_the_fused_op_by_name():
+    lin = nn.Linear(64, 72, specialization="fast_gelu")
+    lin.name_parameter_tensor("ffn")
+    y = lin(Tensor([10, 64], name="x", is_input=True))
+    assert list(y.src_ops())[0]._attrs["op"] == "gemm_rcr_bias_fast_gelu"
+    assert lin.weight.tensor()._attrs["name"] == "ffn_weight"
+    assert nn.Linear(8, 8, bias=False).op._attrs["op"] == "gemm_rcr"
+    with pytest.raises(NotImplementedError):
+        nn.Linear(8, 8, specialization="nope")
+
+
+# ---- registry / target ---------------------------------------------------------------------
+def test_registry_has_every_hook_for_every_op():
+    detect_target()  # importing the ROCm backend registers the hooks
+    for op in ("gemm_rcr", "gemm_rcr_bias", "gemm_rcr_bias_relu", "gemm_rcr_bias_gelu", "gemm_rcr_bias_fast_gelu",
+               "gemm_rcr_bias_add", "gemm_rcr_bias_add_add", "bmm_rcr", "bmm_softmax_bmm_permute",
+               "bmm_softmax_bmm_permute_causal"):
+        for hook in ("config", "filter", "gen_profiler", "gen_function", "func_decl", "func_call"):
+            assert registry.exists(f"rocm.{op}.{hook}"), f"rocm.{op}.{hook}"
+    with pytest.raises(RuntimeError):
+        registry.reg("rocm.gemm_rcr.config", lambda: None)
+    with pytest.raises(RuntimeError):
+        registry.get("rocm.nope.config")
+
+
+def test_target_properties():
+    t = detect_target()
+    assert t.name() == "rocm" and t.src_extension() == ".cpp" and t.dev_select_flag() == "HIP_VISIBLE_DEVICES"
+    assert "{target}" in t.compile_cmd(False) and "{src}" in t.compile_cmd(True)
+    names = ["gemm_rcr_f16_256x256x32_w2x2_dma4_o1_p1_m32_c0", "gemm_rcr_f16_64x64x64_w2x2_v8",
+             "gemm_rcr_f16_128x128x64_w2x2_v8"]
+    assert t.select_minimal_algo(names) == "gemm_rcr_f16_64x64x64_w2x2_v8"
+    from aitemplate_amd.backend.rocm.target_def import ROCM
+
+    with pytest.raises(RuntimeError):
+        ROCM(arch="gfx90a")
+    with t:
+        from aitemplate_amd.backend.target import Target
+
+        assert Target.current() is t
+    with pytest.raises(RuntimeError):
+        Target.current()
+
+
+# ---- profiling plumbing ----------------------------------------------------------------
+def test_profiler_command_line_and_instance_filter(tmp_path, monkeypatch):
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    Y = _gemm_bias_graph(Ms=(4096,), N=4, K=4)
+    op = list(Y.src_ops())[0]
+    with detect_target():
+        res = op.gen_profiler(str(tmp_path), DynamicProfileStrategy.MAX)
+        assert len(res) == 1 and os.access(res[0][1], os.X_OK)
+        assert res[0][1] == os.path.join(str(tmp_path), "profiler", "gemm_rcr_bias", op._get_profiler_filename())
+        # K = 4 leaves only the narrow-load instances
+        assert op._attrs["op_instance"] and all("_v8" not in n and "dma" not in n for n in op._attrs["op_instance"])
+        cmd = op._gen_profile_cmd(os.path.dirname(res[0][1]), op._get_profiler_filename(),
+                                  "M == 4096 && N == 4 && K == 4")
+        assert cmd[1:] == ["gemm", "gemm_rcr_bias", "0", "4096", "4", "4"]
+        op.profile(None, str(tmp_path))
+        assert op._attrs["exec_path"]["M == 4096 && N == 4 && K == 4"].algo in op._attrs["op_instance"]
+    a = ops.bmm_softmax_bmm_permute(shape=(8,), scale=0.5)
+    a(Tensor([16, 64, 40]), Tensor([16, 64, 40]), Tensor([16, 64, 40]))
+    with detect_target():
+        res = a.gen_profiler(str(tmp_path), DynamicProfileStrategy.MAX)
+        key = list(a._attrs["exec_path"])[0]
+        cmd = a._gen_profile_cmd(os.path.dirname(res[0][1]), a._get_profiler_filename(), key)
+        assert cmd[1:] == ["attn", "bmm_softmax_bmm_permute", "0", "16", "64", "64", "40", "40", "8"]
+
+
+def test_extract_profile_result():
+    out = "noise\nOP:tile_a,TIME:0.25,WS:0\nOP:tile_b,TIME:0.125,WS:102400\n"
+    best, failed = extract_profile_result(out)
+    assert not failed and best.op_config == "tile_b" and best.duration == 0.125 and best.workspace == 102400
+    both, failed = extract_profile_result(out, return_ops=["tile_a", "tile_b", "tile_c"])
+    assert [r.op_config for r in both] == ["tile_a", "tile_b"]
+    _, failed = extract_profile_result("segfault")
+    assert failed
+
+
+class _Delegate:
+    def __init__(self):
+        self.results = [None] * 42
+        self.post = False
+
+    def add_result(self, idx, val):
+        sleep(random() * 0.005)
+        self.results[idx] = val
+
+    def postprocess_results(self):
+        assert all(v is not None for v in self.results)
+        self.post = True
+
+
+def test_profiler_runner_with_fake_commands():
+    delegate = _Delegate()
+    pr = ProfilerRunner(devices=[str(i) for i in range(12)], timeout=60, postprocessing_delegate=delegate)
+    for i in range(len(delegate.results)):
+        pr.push(cmds=["sleep", "0"], process_result_callback=(lambda idx: (lambda result, d: d.add_result(idx, 0)))(i))
+    pr.join()
+    assert delegate.post
+
+
+def test_profiler_runner_parses_output_and_picks_fastest(tmp_path):
+    from aitemplate_amd.compiler.base import ExecItem
+    from aitemplate_amd.compiler.ops.gemm_universal.gemm_common import GemmProfilerPostprocessingDelegate
+
+    fake = tmp_path / "fake_profiler.sh"
+    fake.write_text("#!/bin/sh\necho \"device=$HIP_VISIBLE_DEVICES\"\necho OP:tile_a,TIME:0.50,WS:0\necho OP:tile_b,TIME:0.25,WS:0\n"
+                    "echo OP:tile_not_listed,TIME:0.01,WS:0\n")
+    fake.chmod(fake.stat().st_mode | stat.S_IEXEC)
+    attrs = {"op": "gemm_rcr", "exec_path": {"M == 1 && N == 2 && K == 3": ExecItem("k", "c", "")}, "workspace": 0,
+             "split_k": 1, "op_instance": {"tile_a": 0, "tile_b": 1}}
+    pr = ProfilerRunner(devices=["0"], postprocessing_delegate=GemmProfilerPostprocessingDelegate(), timeout=30)
+    pr.push([str(fake)], func_attrs=attrs, profiler_filename="x", exec_key="M == 1 && N == 2 && K == 3", split_k=1)
+    pr.join()
+    assert attrs["exec_path"]["M == 1 && N == 2 && K == 3"].algo == "tile_b"
+    bad = ProfilerRunner(devices=["0"], postprocessing_delegate=GemmProfilerPostprocessingDelegate(), timeout=30)
+    bad.push(["false"], func_attrs=attrs, profiler_filename="x", exec_key="M == 1 && N == 2 && K == 3", split_k=1)
+    with pytest.raises(RuntimeError, match="Profil"):
+        bad.join()
+
+
+# ---- passes and code generation ----------------------------------------------------------------
+def test_naming_aliases_and_memory_planning():
+    reset_name_counters()
+    X = Tensor([8, 16], name="x", is_input=True)
+    W1, W2 = Tensor([32, 16], name="w1"), Tensor([24, 32], name="w2")
+    h = ops.gemm_rcr()(X, W1)
+    y = ops.gemm_rcr()(h, W2)
+    y._attrs["is_output"] = True
+    y._attrs["name"] = "out"
+    graph = transform.toposort(y)
+    assert [t._attrs["name"] for t in graph][-1] == "out"
+    transform.name_graph(graph)
+    transform.mark_param_tensor(graph, [y])
+    names = [t._attrs["name"] for t in graph]
+    assert "gemm_rcr_0_0" in names and h._attrs["name"] == "gemm_rcr_0_0"
+    assert [op._attrs["name"] for op in transform.get_sorted_ops(graph)] == ["gemm_rcr_0", "gemm_rcr_1"]
+    assert h._attrs["shape"][0]._attrs["name"] == "x_dim_0"  # dim objects are shared and named once
+    assert W1._attrs["is_param"] and not h._attrs["is_param"]
+    blob, ws = transform.memory_planning(graph)
+    assert h._attrs["offset"] == 0 and blob == 8 * 32 * 2 and ws == 0
+    # attention: the op's [B, M, O] tensor lives in the reshaped output's buffer
+    a = ops.bmm_softmax_bmm_permute(shape=(2,), scale=1.0)
+    o = a(Tensor([4, 8, 16], name="q", is_input=True), Tensor([4, 8, 16], name="k", is_input=True),
+          Tensor([4, 8, 16], name="v", is_input=True))
+    o._attrs["is_output"] = True
+    o._attrs["name"] = "o"
+    g2 = transform.toposort(o)
+    transform.name_graph(g2)
+    transform.mark_param_tensor(g2, [o])
+    inner = a._attrs["outputs"][0]
+    assert inner._attrs["external_tensor"] is o and inner._attrs["has_output_aliases"]
+    assert transform.memory_planning(g2) == (0, 0)
+
+
+def test_compile_model_builds_a_library_exporting_the_whole_abi(tmp_path, monkeypatch):
+    """No GPU here: creating the container fails cleanly, but sources are generated, the
+    library links and exports every function include/model_interface.h declares."""
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    Y = _gemm_bias_graph(Ms=(1, 128), N=64, K=1024, op="gemm_rcr_bias_fast_gelu")
+    import torch
+
+    if torch.cuda.is_available():
+        compile_model(Y, detect_target(), str(tmp_path), "abi_check").close()
+    else:
+        with pytest.raises(RuntimeError, match="AITemplateModelContainerCreate"):
+            compile_model(Y, detect_target(), str(tmp_path), "abi_check")
+    build = tmp_path / "abi_check"
+    src = (build / "gemm_rcr_bias_fast_gelu_0.cpp").read_text()
+    assert "void gemm_rcr_bias_fast_gelu_0(void* in_ptr, void* weight_ptr, void* out_ptr, void* bias_ptr, " \
+           "int64_t* a_dim0, int64_t* a_dim1, int64_t* b_dim0, int64_t* b_dim1, int64_t* c_dim0, int64_t* c_dim1, " \
+           "hipStream_t stream)" in src
+    assert "if (M >= 1 && M <= 128 && N == 64 && K == 1024)" in src
+    assert "aitamd_gemm_rcr(3, 0, algo" in src and "Unsupported workload" in src
+    model_src = (build / "model-generated.cpp").read_text()
+    assert "ParamDim(1, 128, &m)" in model_src and 'OpEntry{"gemm_rcr_bias_fast_gelu_0"' in model_src
+    header = open(os.path.join(ROOT, "include", "model_interface.h")).read()
+    declared = sorted(set(re.findall(r"AIT_EXPORT AITemplateError\s+(AITemplate\w+)\s*\(", header)))
+    assert len(declared) == 32, declared
+    out = subprocess.run(["nm", "-D", "--defined-only", str(build / "test.so")], capture_output=True, text=True).stdout
+    exported = sorted(set(re.findall(r" T (AITemplate\w+)", out)))
+    assert exported == declared
+    # nothing else leaks out of the model library except the C ABI
+    others = [l.split()[-1] for l in out.splitlines() if " T " in l and "AITemplate" not in l]
+    assert not [s for s in others if not s.startswith("_")], others
