@@ -23,6 +23,14 @@ if ROOT not in sys.path:
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch of the headline workload, per kernel instance, from two counter runs of
+# this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter read for the
+# 256 MiB copy of --copy-probe in the same run.  Instances never measured report null.
+MEASURED_TRAFFIC_BYTES = {
+    # FETCH_SIZE 95421.4 KiB x 2.000 (copy: 131084.6 read for 262144 KiB) + WRITE_SIZE 147456 KiB x 1.000
+    "gemm_rcr_f16_256x256x32_w2x4_dma4_o1_p1_m32_c0": 346_412_000,
+}
+
 SHAPES = {
     # name: (op, M, N, K, residuals)
     "c1": ("gemm_rcr_bias", 256, 1024, 1024, 0),
@@ -72,6 +80,33 @@ def time_gemm(torch, eager, name, steps, warmup, algo=-1):
             "flops": 2 * M * N * K, "bytes": 2 * (M * K + N * K + N + (1 + nres) * M * N)}
 
 
+def pick_instance(torch, eager, kernels, name, iters=15):
+    """Untimed selection pass, the same procedure compile_model's profiling step applies
+    (python/aitemplate/compiler/ops/gemm_universal/gemm_common.py:743-829 in the reference):
+    time every instance that supports the problem and keep the fastest."""
+    op, M, N, K, nres = SHAPES[name]
+    epi = kernels.EPILOGUE_OF_OP[op]
+    lib = kernels.load()
+    best, best_ms = -1, float("inf")
+    for algo in range(lib.aitamd_gemm_num_algos(epi, 0)):
+        if not lib.aitamd_gemm_algo_supported(epi, 0, algo, M, N, K, K, K, 16):
+            continue
+        ms = time_gemm(torch, eager, name, iters, 3, algo)["event_ms_per_launch"]
+        if ms < best_ms:
+            best, best_ms = algo, ms
+    return best
+
+
+def copy_probe(torch, nbytes=256 << 20, reps=5):
+    """A plain device copy of known size, for scaling the FETCH_SIZE / WRITE_SIZE counters of a
+    counter-collection run of this script (the copy reads nbytes and writes nbytes per launch)."""
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(reps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
+
 def cpu_baseline(torch, max_seconds=20.0):
     """The oracle expression of the headline config in fp32 on the host cores."""
     from oracle import oracle
@@ -104,7 +139,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--algo", type=int, default=-1, help="kernel instance index (-1: library heuristic)")
+    ap.add_argument("--algo", type=int, default=-1, help="kernel instance index (-1: see --select)")
+    ap.add_argument("--select", choices=("profile", "heuristic"), default="profile",
+                    help="how the kernel instance is chosen when --algo is not given: an untimed profiling "
+                         "pass over all instances (what compile_model does) or the library's heuristic")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch a 256 MiB device copy 5 times (counter calibration for profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--all-configs", action="store_true", help="also time the other GEMM configurations")
     args = ap.parse_args()
@@ -122,11 +162,18 @@ def main():
         sys.exit(2)
     _kernels.load()
 
-    r = time_gemm(torch, eager, "c2a", args.steps, args.warmup, args.algo)
+    op, M, N, K, _ = SHAPES["c2a"]
+    algo = args.algo
+    if algo < 0 and args.select == "profile":
+        algo = pick_instance(torch, eager, _kernels, "c2a")
+    if algo < 0:
+        algo = _kernels.load().aitamd_gemm_heuristic_algo(3, 0, 1, M, N, K, K, K, 16)
+    if args.copy_probe:
+        copy_probe(torch)
+    r = time_gemm(torch, eager, "c2a", args.steps, args.warmup, algo)
     tflops = r["flops"] / (r["wall_ms_per_step"] * 1e-3) / 1e12
     achieved = r["flops"] / (r["event_ms_per_launch"] * 1e-3) / 1e12
-    op, M, N, K, _ = SHAPES["c2a"]
-    algo = args.algo if args.algo >= 0 else _kernels.load().aitamd_gemm_heuristic_algo(3, 0, 1, M, N, K, K, K, 16)
+    instance = _kernels.gemm_algo_names(3, 0)[algo]
     line = {
         "metric": "TFLOP/s + % fp16 MFMA peak, gemm_rcr_bias_gelu M=24576 K=768 N=3072",
         "value": round(tflops, 2),
@@ -143,9 +190,10 @@ def main():
         "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
         "config": {"workload": "configs[1]: gemm_rcr_bias_gelu fp16 X[24576,768] W[3072,768] bias[3072], "
                                "fp32 accumulate, tanh-GELU fused, inputs resident in HBM, rotating operand sets",
-                   "instance": _kernels.gemm_algo_names(3, 0)[algo]},
+                   "instance": instance, "instance_index": algo,
+                   "instance_selected_by": "--algo" if args.algo >= 0 else args.select},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": None},
+                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(instance)},
     }
     if args.all_configs:
         others = {}
