@@ -42,7 +42,7 @@ SHAPES = {
 
 def _make_pool(torch, op, M, N, K, nres, pool_bytes=600 << 20):
     set_bytes = 2 * (M * K + N * K + N + (1 + nres) * M * N)
-    sets = max(2, min(16, pool_bytes // set_bytes + 1))
+    sets = max(2, min(16, pool_bytes // set_bytes + 1)) if pool_bytes else 1
     g = torch.Generator(device="cuda").manual_seed(1)
     pool = []
     for _ in range(sets):
@@ -107,6 +107,31 @@ def copy_probe(torch, nbytes=256 << 20, reps=5):
     torch.cuda.synchronize()
 
 
+def in_abi(torch, count=100):
+    """The same workload through the whole product path: ops.gemm_rcr_bias_gelu -> compile_model
+    (instance chosen by the prebuilt profiler program) -> AITemplateModelContainerBenchmark.
+    One fixed operand set, as a serving loop would hold it."""
+    import tempfile
+
+    from aitemplate_amd.compiler import compile_model, ops
+    from aitemplate_amd.compiler.base import Tensor
+    from aitemplate_amd.testing import detect_target
+
+    op, M, N, K, _ = SHAPES["c2a"]
+    X = Tensor([M, K], name="input_0", is_input=True)
+    W = Tensor([N, K], name="input_1", is_input=True)
+    B = Tensor([N], name="input_2", is_input=True)
+    Y = getattr(ops, op)()(X, W, B)
+    Y._attrs["name"], Y._attrs["is_output"] = "output_0", True
+    (x, w, b, _, out), = _make_pool(torch, op, M, N, K, 0, pool_bytes=0)[:1]
+    with tempfile.TemporaryDirectory(prefix="aitamd_bench_") as tmp:
+        with compile_model(Y, detect_target(), tmp, "bench_c2a") as module:
+            module.benchmark_with_tensors([x, w, b], [out], count=10)
+            ms, _, _ = module.benchmark_with_tensors([x, w, b], [out], count=count)
+    return {"ms_per_run": round(ms, 5), "tflops": round(2 * M * N * K / (ms * 1e-3) / 1e12, 2),
+            "via": f"compile_model + AITemplateModelContainerBenchmark, count={count}, one fixed operand set"}
+
+
 def cpu_baseline(torch, max_seconds=20.0):
     """The oracle expression of the headline config in fp32 on the host cores."""
     from oracle import oracle
@@ -146,6 +171,7 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a 256 MiB device copy 5 times (counter calibration for profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-in-abi", action="store_true", help="skip the compile_model + container Benchmark leg")
     ap.add_argument("--all-configs", action="store_true", help="also time the other GEMM configurations")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -203,6 +229,8 @@ def main():
             others[name] = {"op": SHAPES[name][0], "ms": round(o["event_ms_per_launch"], 5),
                             "tflops": round(o["flops"] / t / 1e12, 2), "gbs": round(o["bytes"] / t / 1e9, 1)}
         line["other_configs"] = others
+    if not args.no_in_abi:
+        line["in_abi"] = in_abi(torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(line))
