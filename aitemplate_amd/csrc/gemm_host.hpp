@@ -18,7 +18,7 @@ struct GemmAlgo {
   int kvec;
   int lds_bytes;
   int wgs_per_cu;  // workgroups of this instance one CU holds at once
-  int direct_lds;  // 1: direct-to-LDS ring pipeline, 0: register-staged loads
+  int direct_lds;  // 0: register-staged loads, 1: direct-to-LDS ring, 2: persistent direct-to-LDS ring
   hipError_t (*launch)(const GemmParams& p, hipStream_t stream);
 };
 

@@ -6,6 +6,7 @@
 
 #include "gemm_host.hpp"
 #include "gemm_kernel_dma.hpp"
+#include "gemm_kernel_persist.hpp"
 
 #ifndef AITAMD_EPI
 #error "compile with -DAITAMD_EPI=<id>"
@@ -39,6 +40,30 @@ struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>> {
       gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, Epi>;
 };
 
+template <int BM, int BN, int BK, int WM, int WN, int NS>
+struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS>> {
+  static constexpr auto value = gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS>, Epi>;
+};
+template <class Tile>
+struct IsPersistent {
+  static constexpr bool value = false;
+};
+template <int BM, int BN, int BK, int WM, int WN, int NS>
+struct IsPersistent<GemmTilePersist<BM, BN, BK, WM, WN, NS>> {
+  static constexpr bool value = true;
+};
+
+// compute units of a device (looked up once per device)
+inline int device_cus(int dev) {
+  static int cus[kMaxDevices] = {};
+  int v = cus[dev % kMaxDevices];
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cus[dev % kMaxDevices] = v;
+  }
+  return v;
+}
+
 template <class Tile>
 hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
   auto kernel = KernelOf<Tile>::value;
@@ -61,6 +86,13 @@ hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
   if (tiles <= 0 || p.batch <= 0) return hipSuccess;
   if (tiles > 0x7fffffffll) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, (unsigned)(p.batch < 65535 ? p.batch : 65535), 1);
+  if constexpr (IsPersistent<Tile>::value) {
+    // one workgroup per CU walks (tile, batch) pairs
+    const int64_t total = tiles * p.batch;
+    if (total > 0x7fffffffll) return hipErrorInvalidValue;
+    const int cus = device_cus(dev);
+    grid = dim3((unsigned)(total < cus ? total : cus), 1, 1);
+  }
   hipLaunchKernelGGL(kernel, grid, dim3(Tile::NT), Tile::kLdsBytes, stream, p);
   return hipGetLastError();
 }
@@ -101,9 +133,14 @@ const GemmAlgo kAlgos[] = {
    dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::NT, OCC,                        \
                   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kLdsBytes),                      \
    1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>},
+#define AITAMD_GEMM_TILE_PERSIST(BM, BN, BK, WM, WN, NS)                                                  \
+  {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_persist" #NS,                      \
+   BM, BN, BK, GemmTilePersist<BM, BN, BK, WM, WN, NS>::NT, 8, GemmTilePersist<BM, BN, BK, WM, WN, NS>::kLdsBytes, \
+   1, 2, &launch_tile<GemmTilePersist<BM, BN, BK, WM, WN, NS>>},
 #include "gemm_tiles.inc"
 #undef AITAMD_GEMM_TILE
 #undef AITAMD_GEMM_TILE_DMA
+#undef AITAMD_GEMM_TILE_PERSIST
 };
 
 }  // namespace

@@ -1,0 +1,316 @@
+// Persistent variant of the direct-to-LDS RCR GEMM: one workgroup per CU walks its
+// tiles and the LDS ring never drains.
+//
+// gemm_rcr_dma_kernel starts every tile cold: the first K-slab needs a full trip to
+// memory (about 6 k cycles per 256x256 tile on MI355X) before the first MFMA
+// can issue, which is a tenth of a BERT-FFN-sized tile (K = 768).  Here the slab
+// stream runs across tile boundaries - while a tile's epilogue runs, the first
+// slabs of the workgroup's next tile are already landing - so only the first
+// tile of a workgroup pays the fill.
+//
+// Main loop: as gemm_rcr_dma_kernel with PIPE = 1 (barrier inside the last MFMA
+// step of a slab, first fragments of the next slab prefetched across it, loads
+// issued in two portions per slab).
+//
+// Epilogue: the accumulators are rounded to the output type, transposed through a
+// wave-private LDS strip outside the ring (32 rows at a time, 16-byte chunks XOR-
+// swizzled, conflict-free both ways), read back as 8 consecutive columns per lane,
+// combined with bias / residuals in fp32 and stored with 16-byte stores.  Rounding
+// the accumulator before the element-wise functor is what the reference's
+// Composable-Kernel path does too (C-shuffle to the C type, then the functor;
+// python/aitemplate/utils/mk_ck_lib/gemm_operation.py:487).
+#pragma once
+
+#include "gemm_kernel_dma.hpp"
+
+namespace aitamd {
+
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_>
+struct GemmTilePersist {
+  static constexpr int MT = 32, KSTEP = 16, QN = 2, ACC_N = 16;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_;
+  static constexpr int WGM = WGM_, WGN = WGN_, NS = NS_;
+  static constexpr int NW = WGM * WGN;
+  static constexpr int NT = NW * kWaveSize;
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  static constexpr int MI = WTM / MT, NI = WTN / MT;
+  static constexpr int KK = BK / KSTEP;
+  static constexpr int CPR = BK / 8;
+  static constexpr int RPW = (256 / (BK * 2)) > 0 ? (256 / (BK * 2)) : 1;
+  static constexpr int ROWS_PER_LOAD = 64 / CPR;
+  static constexpr int A_LOADS = BM / ROWS_PER_LOAD;
+  static constexpr int B_LOADS = BN / ROWS_PER_LOAD;
+  static constexpr int LOADS_PER_STEP = (A_LOADS + B_LOADS) / NW;  // wave-loads per slab per wave
+  static constexpr int L_P0 = (LOADS_PER_STEP + 1) / 2;            // issued in a slab's last step
+  static constexpr int STAGE_ELEMS = (BM + BN) * BK;
+  static constexpr int RING_BYTES = NS * STAGE_ELEMS * 2;
+  // wave-private epilogue strip: 32 rows x WTN elements of the output type
+  static constexpr int STRIP_CHUNKS = WTN / 8;  // 16-byte chunks per strip row
+  static constexpr int STRIP_PITCH = WTN * 2;
+  static constexpr int STRIP_BYTES = MT * STRIP_PITCH;
+  static constexpr int ROWS_PER_PASS = 64 / STRIP_CHUNKS;
+  static constexpr int PASSES = MT / ROWS_PER_PASS;
+  static constexpr int kLdsBytes = RING_BYTES + NW * STRIP_BYTES;
+  static_assert(KK == 2, "two MFMA steps per slab");
+  static_assert(NS >= 4, "needs one slab in flight behind the one being waited for");
+  static_assert((A_LOADS + B_LOADS) % NW == 0, "slab loads must divide over the waves");
+  static_assert(STRIP_CHUNKS == 4 || STRIP_CHUNKS == 8 || STRIP_CHUNKS == 16, "strip swizzle needs 2^k chunks");
+  static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
+};
+
+template <class T, class Tile, class Epi>
+__global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const GemmParams p) {
+  using Tr = ElemTraits<T>;
+  using vec8 = typename Tr::vec8;
+  using Mfma = MfmaOp<T, 32>;
+  using acc_t = typename Mfma::acc_t;
+  constexpr int BM = Tile::BM, BN = Tile::BN, BK = Tile::BK, NS = Tile::NS;
+  constexpr int MI = Tile::MI, NI = Tile::NI, MT = 32;
+  constexpr int L = Tile::LOADS_PER_STEP, L_P0 = Tile::L_P0;
+  constexpr int SC = Tile::STRIP_CHUNKS;
+  typedef __attribute__((address_space(3))) void lds_void;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* const smem = reinterpret_cast<T*>(smem_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Tile::WGN;
+  const int wn = wave % Tile::WGN;
+  const int fr = lane & 31;
+  const int fq = lane >> 5;
+  unsigned char* const strip = smem_raw + Tile::RING_BYTES + wave * Tile::STRIP_BYTES;
+
+  const int tiles_per_batch = p.tiles_m * p.tiles_n;
+  const int total_tiles = tiles_per_batch * p.batch;
+  const int G = gridDim.x;
+  const int g = blockIdx.x;
+  const int my_tiles = (total_tiles - g + G - 1) / G;
+  const int k_tiles = (p.K + BK - 1) / BK;
+
+  // ---- loader: a stream of slabs that runs across this workgroup's tiles ------------------------
+  const int l_row = lane / Tile::CPR;
+  const int l_slot = lane % Tile::CPR;
+  uint32_t l_off[L];
+  int l_chunk_k[L];
+#pragma unroll
+  for (int i = 0; i < L; ++i) {
+    const int j = wave + i * Tile::NW;
+    const bool is_a = j < Tile::A_LOADS;
+    const int row = (is_a ? j : j - Tile::A_LOADS) * Tile::ROWS_PER_LOAD + l_row;
+    const int chunk = l_slot ^ ((row / Tile::RPW) % Tile::CPR);
+    l_off[i] = (uint32_t)(((int64_t)row * (is_a ? p.lda : p.ldb) + chunk * 8) * 2);
+    l_chunk_k[i] = chunk * 8;
+  }
+
+  struct TileCoord {
+    int m0, n0, batch;
+  };
+  auto tile_coord = [&](int i) {
+    TileCoord c;
+    const int v = g + i * G;
+    const int b = v / tiles_per_batch;
+    const int t = v - b * tiles_per_batch;
+    int tm, tn;
+    map_tile<8>(t, p.tiles_m, p.tiles_n, tm, tn);
+    c.m0 = tm * BM;
+    c.n0 = tn * BN;
+    c.batch = b;
+    return c;
+  };
+
+  int ld_i = 0, ld_kt = 0, ld_stage = 0;
+  __amdgpu_buffer_rsrc_t ra, rb;
+  auto set_loader_tile = [&](int i) {
+    if (i < my_tiles) {
+      const TileCoord c = tile_coord(i);
+      const int rows_a = (p.M - c.m0) < BM ? (p.M - c.m0) : BM;
+      const int rows_b = (p.N - c.n0) < BN ? (p.N - c.n0) : BN;
+      const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)c.batch * p.sa + (int64_t)c.m0 * p.lda;
+      const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)c.batch * p.sb + (int64_t)c.n0 * p.ldb;
+      ra = make_rsrc(Ab, clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2));
+      rb = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
+    } else {
+      // past the last tile the ring keeps turning on zero-sized buffers: every lane is out of
+      // range, nothing is fetched, and the number of loads in flight per step stays constant
+      ra = make_rsrc(p.a, 0);
+      rb = make_rsrc(p.b, 0);
+    }
+  };
+  set_loader_tile(0);
+
+  // Issue wave-loads [i0, i1) of the stream's current slab; the portion that ends the slab
+  // advances the stream to the next slab (and tile).
+  auto issue_part = [&](int i0, int i1) {
+    const int k0 = ld_kt * BK;
+    T* sbase = smem + ld_stage * Tile::STAGE_ELEMS;
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+      if (i < i0 || i >= i1) continue;
+      const int j = wave + i * Tile::NW;
+      const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + (uint32_t)(k0 * 2) : kOobOffset;
+      T* dst = sbase + j * 512;  // 1 KiB per wave-load; A blocks then B blocks
+      if (j < Tile::A_LOADS)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)dst, 16, off, 0, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)dst, 16, off, 0, 0, 0);
+    }
+    if (i1 < L) return;
+    ld_stage = ld_stage + 1 == NS ? 0 : ld_stage + 1;
+    if (++ld_kt == k_tiles) {
+      ld_kt = 0;
+      ++ld_i;
+      set_loader_tile(ld_i);
+    }
+  };
+
+  // ---- fragments ------------------------------------------------------------------------------
+  int a_rd[2], b_rd[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    a_rd[kk] = dma_lds_chunk_elem<Tile>(wm * Tile::WTM + fr, kk * 2 + fq);
+    b_rd[kk] = BM * BK + dma_lds_chunk_elem<Tile>(wn * Tile::WTN + fr, kk * 2 + fq);
+  }
+  auto load_frags = [&](const T* st, int kk, vec8* af, vec8* bf) {
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[kk] + mi * MT * BK);
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) bf[ni] = *reinterpret_cast<const vec8*>(st + b_rd[kk] + ni * MT * BK);
+  };
+  acc_t acc[MI][NI];
+  vec8 af[2][MI], bf[2][NI];
+  // operands swapped: the MFMA produces the transposed block, so a lane holds 4 consecutive
+  // output columns of one row
+  auto mfmas = [&](const vec8* a, const vec8* b) {
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = Mfma::run(b[ni], a[mi], acc[mi][ni]);
+  };
+  auto mfmas_first = [&](const vec8* a, const vec8* b) {
+    const acc_t zero = {};
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = Mfma::run(b[ni], a[mi], zero);
+  };
+
+  // ---- epilogue -------------------------------------------------------------------------------
+  const T* bias = reinterpret_cast<const T*>(p.bias);
+  bool vec_ok = ((p.N & 7) == 0) && ((p.ldc & 7) == 0) && ((p.sc & 7) == 0) &&
+      ((reinterpret_cast<uintptr_t>(p.c) & 15) == 0);
+  if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
+  if (Epi::kNumD >= 1)
+    vec_ok = vec_ok && ((p.ldd & 7) == 0) && ((p.sd & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 15) == 0);
+  if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 15) == 0);
+  // strip addressing: row r, 16-byte chunk c lives at r * PITCH + ((c ^ (r % SC)) << 4)
+  const int w_base = fr * Tile::STRIP_PITCH + fq * 8;
+  const int w_swz = fr & (SC - 1);
+  const int r_row = lane / SC;
+  const int r_c = lane % SC;
+
+  auto epilogue = [&](const TileCoord& c) {
+    T* Cb = reinterpret_cast<T*>(p.c) + (int64_t)c.batch * p.sc;
+    const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)c.batch * p.sd : nullptr;
+    const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)c.batch * p.sd : nullptr;
+    const int n = c.n0 + wn * Tile::WTN + r_c * 8;  // the lane's 8 columns: the same in every pass
+    vec8 bv = {};
+    if constexpr (Epi::kHasBias) {
+      if (vec_ok && n < p.N) bv = *reinterpret_cast<const vec8*>(bias + n);
+    }
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          typename Tr::vec4 h;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) h[j] = Tr::from_float(acc[mi][ni][gq * 4 + j]);
+          *reinterpret_cast<u32x2*>(strip + w_base + (((ni * 4 + gq) ^ w_swz) << 4)) = __builtin_bit_cast(u32x2, h);
+        }
+      // the strip is private to the wave and LDS executes one wave's accesses in order
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int ps = 0; ps < Tile::PASSES; ++ps) {
+        const int row = ps * Tile::ROWS_PER_PASS + r_row;
+        const vec8 raw =
+            *reinterpret_cast<const vec8*>(strip + row * Tile::STRIP_PITCH + ((r_c ^ (row & (SC - 1))) << 4));
+        const int m = c.m0 + wm * Tile::WTM + mi * MT + row;
+        if (m < p.M && n < p.N) {
+          const int64_t c_idx = (int64_t)m * p.ldc + n;
+          const int64_t d_idx = (int64_t)m * p.ldd + n;
+          if (vec_ok) {
+            vec8 d0v = {}, d1v = {};
+            if constexpr (Epi::kNumD >= 1) d0v = *reinterpret_cast<const vec8*>(D0b + d_idx);
+            if constexpr (Epi::kNumD >= 2) d1v = *reinterpret_cast<const vec8*>(D1b + d_idx);
+            vec8 o;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              o[j] = Tr::from_float(Epi::apply(Tr::to_float(raw[j]), Tr::to_float(bv[j]), Tr::to_float(d0v[j]),
+                                               Tr::to_float(d1v[j])));
+            *reinterpret_cast<vec8*>(Cb + c_idx) = o;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              if (n + j < p.N) {
+                float bj = 0.f, d0j = 0.f, d1j = 0.f;
+                if constexpr (Epi::kHasBias) bj = Tr::to_float(bias[n + j]);
+                if constexpr (Epi::kNumD >= 1) d0j = Tr::to_float(D0b[d_idx + j]);
+                if constexpr (Epi::kNumD >= 2) d1j = Tr::to_float(D1b[d_idx + j]);
+                Cb[c_idx + j] = Tr::from_float(Epi::apply(Tr::to_float(raw[j]), bj, d0j, d1j));
+              }
+            }
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  };
+
+  // ---- prologue: slabs 0 .. NS-3 whole, slab NS-2 up to its first portion -------------------------
+#pragma unroll
+  for (int s = 0; s < NS - 2; ++s) issue_part(0, L);
+  issue_part(0, L_P0);
+  wait_vmcnt<(NS - 3) * L + L_P0>();
+  __builtin_amdgcn_s_barrier();
+  int rd_stage = 0;
+  load_frags(smem, 0, af[0], bf[0]);
+
+  for (int i = 0; i < my_tiles; ++i) {
+    const TileCoord cur = tile_coord(i);
+    for (int kt = 0; kt < k_tiles; ++kt) {
+      const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
+      const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
+      const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
+      // first step: the rest of the slab whose first portion went out in the previous step
+      issue_part(L_P0, L);
+      load_frags(cur_st, 1, af[1], bf[1]);
+      if (kt == 0)
+        mfmas_first(af[0], bf[0]);
+      else
+        mfmas(af[0], bf[0]);
+      sched_step<MI * NI, MI + NI, L - L_P0>();
+      // last step: the next slab has landed once at most (NS-3) younger slabs are in flight; past
+      // the barrier nobody reads the previous slab any more, so its ring slot starts taking a new
+      // slab, and the next slab's first fragments are fetched under this slab's last MFMAs
+      wait_vmcnt<(NS - 3) * L>();
+      __builtin_amdgcn_s_barrier();
+      issue_part(0, L_P0);
+      load_frags(nxt_st, 0, af[0], bf[0]);
+      mfmas(af[1], bf[1]);
+      sched_step<MI * NI, MI + NI, L_P0>();
+      rd_stage = nx_stage;
+    }
+    epilogue(cur);
+  }
+  // no LDS-DMA may be in flight into a workgroup that has ended
+  wait_vmcnt<0>();
+}
+
+}  // namespace aitamd
