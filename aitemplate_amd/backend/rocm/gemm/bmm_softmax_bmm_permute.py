@@ -11,7 +11,7 @@ from ...target import Target
 from . import common
 
 _OPS = ("bmm_softmax_bmm_permute", "bmm_softmax_bmm_permute_causal")
-_INSTANCE = "attention_q128_kv64"
+_INSTANCE = "attention_q128"
 
 
 def _config(func_attrs, dtype="float16"):

@@ -2,8 +2,8 @@
 // folded into the store (bmm_softmax_bmm_permute), gfx950.
 //
 // The score matrix never leaves the chip.  One wave owns 32 query rows and walks
-// the keys/values in blocks of 32; a workgroup of 4 waves shares each 64-row
-// K / V tile through LDS.
+// the keys/values in blocks of 32; a workgroup of 4 waves shares each 64- or
+// 128-row K / V tile through LDS.
 //
 //  * S^T = K Q^T is computed with v_mfma_f32_32x32x16 (K tile rows as the A
 //    operand, the wave's Q rows - kept in registers for the whole kernel - as
@@ -37,14 +37,14 @@ struct AttnParams {
   int32_t causal;
 };
 
-template <int KS_, int OT_>
+template <int KS_, int OT_, int BN_ = ((16 * KS_ + 32 * OT_) <= 112 ? 128 : 64)>
 struct AttnTile {
   static constexpr int KS = KS_;          // K padded to 16 * KS
   static constexpr int OT = OT_;          // O padded to 32 * OT
   static constexpr int KP = 16 * KS;
   static constexpr int OP = 32 * OT;
   static constexpr int BM = 128;          // query rows per workgroup (4 waves x 32)
-  static constexpr int BN = 64;           // keys per LDS tile
+  static constexpr int BN = BN_;          // keys per LDS tile: 128 while two workgroups still fit one CU's LDS
   static constexpr int NT = 256;
   static constexpr int K_PITCH = KP + 8;  // halves; keeps 16 consecutive rows on distinct banks
   static constexpr int V_PITCH = OP + 8;
@@ -79,6 +79,10 @@ AITAMD_DEVICE float max_across_halves(float x) {
   // lane l and lane l^32 hold the two halves of one query row
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+AITAMD_DEVICE float min_across_halves(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fminf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 AITAMD_DEVICE float sum_across_halves(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -193,7 +197,11 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
     for (int ot = 0; ot < OT; ++ot)
 #pragma unroll
       for (int e = 0; e < 16; ++e) oacc[ot][e] = 0.0f;
-    float m_run = -INFINITY;  // running max of the scaled scores of this lane's row (log2 domain)
+    // running extremum of the raw scores of this lane's row: the maximum, or the minimum when the
+    // scale is negative (either way the score whose scaled value is largest)
+    const bool neg_scale = p.scale_log2e < 0.0f;
+    const float m_init = neg_scale ? INFINITY : -INFINITY;
+    float m_run = m_init;
     float l_run = 0.0f;       // running sum over this lane's half of the keys
 
     if (n_tiles > 0) {
@@ -220,6 +228,8 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
       for (int blk = 0; blk < BN / 32; ++blk) {
         const int nb = t * BN + blk * 32;  // first key of this 32-key block
         // ---- S^T block: rows = keys, columns = this wave's 32 query rows
+        // (issuing the next block's product ahead of this block's softmax was measured: no gain at
+        // head dim 40 and a quarter slower at head dim 64, where the extra live accumulator costs more)
         f32x16 s;
 #pragma unroll
         for (int e = 0; e < 16; ++e) s[e] = 0.0f;
@@ -228,27 +238,54 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
           const vec8 kf = *reinterpret_cast<const vec8*>(cK + (blk * 32 + r32) * KPI + ks * 16 + h * 8);
           s = Tr::mfma32(kf, qf[ks], s);
         }
-        // lane holds keys nb + 8 g + 4 h + r (element 4 g + r) of query row q_row
-        float tmax = -INFINITY;
+        // lane holds keys nb + 8 g + 4 h + r (element 4 g + r) of query row q_row.
+        // The running maximum is kept on the raw scores (minimum when the scale is negative) and the
+        // scale is folded into the exponent: p = exp2(s * c - m * c) is one FMA and one v_exp per score.
+        // Only blocks that reach past N or touch the causal diagonal pay for masking.
+        const bool need_mask = (nb + 32 > p.N) || (p.causal && nb + 31 > m0 + wave * 32);
+        bool dead[16];
+        if (need_mask) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int n = nb + (e >> 2) * 8 + h * 4 + (e & 3);
-          float v = s[e] * p.scale_log2e;
-          const bool masked = (n >= p.N) || (p.causal && n > q_row);
-          v = masked ? -INFINITY : v;
-          s[e] = v;
-          tmax = fmaxf(tmax, v);
+          for (int e = 0; e < 16; ++e) {
+            const int n = nb + (e >> 2) * 8 + h * 4 + (e & 3);
+            dead[e] = (n >= p.N) || (p.causal && n > q_row);
+          }
         }
-        tmax = max_across_halves(tmax);
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // fully masked so far
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);  // 0 when m_run = -inf
-        float psum = 0.0f;
+        float text = neg_scale ? INFINITY : -INFINITY;
+        if (need_mask) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float pe = __builtin_amdgcn_exp2f(s[e] - m_safe);
-          s[e] = pe;
-          psum += pe;
+          for (int e = 0; e < 16; ++e) {
+            const float v = dead[e] ? m_init : s[e];
+            text = neg_scale ? fminf(text, v) : fmaxf(text, v);
+          }
+        } else if (neg_scale) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) text = fminf(text, s[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) text = fmaxf(text, s[e]);
+        }
+        text = neg_scale ? min_across_halves(text) : max_across_halves(text);
+        const float m_new = neg_scale ? fminf(m_run, text) : fmaxf(m_run, text);
+        const float m_safe = __builtin_isinf(m_new) ? 0.0f : m_new;  // every key so far masked
+        const float c = p.scale_log2e;
+        const float alpha = __builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m_safe) * c);
+        const float mc = -m_safe * c;
+        float psum = 0.0f;
+        if (need_mask) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const float pe = dead[e] ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc));
+            s[e] = pe;
+            psum += pe;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc));
+            s[e] = pe;
+            psum += pe;
+          }
         }
         l_run = l_run * alpha + psum;
         m_run = m_new;

@@ -261,7 +261,7 @@ int profile_attention(int dtype, int64_t B, int64_t M, int64_t N, int64_t K, int
   HIP_OK(hipEventSynchronize(e1));
   float ms = 0.f;
   HIP_OK(hipEventElapsedTime(&ms, e0, e1));
-  printf("OP:attention_q128_kv64,TIME:%.6f,WS:0\n", ms / (iters > 0 ? iters : 1));
+  printf("OP:attention_q128,TIME:%.6f,WS:0\n", ms / (iters > 0 ? iters : 1));
   HIP_OK(hipStreamDestroy(stream));
   return 0;
 }

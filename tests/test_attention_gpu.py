@@ -60,6 +60,13 @@ def test_bf16():
     _check(8, 100, 100, 40, 40, 8, causal=True, dtype=torch.bfloat16, tol=4e-2)
 
 
+@pytest.mark.parametrize("scale", [-0.3, 0.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_negative_and_zero_scale(scale, causal):
+    # the running extremum is kept on raw scores: a negative scale tracks the minimum instead
+    _check(8, 200, 200, 40, 40, 4, causal=causal, scale=scale, seed=9)
+
+
 def test_large_scores_do_not_overflow():
     # scores of magnitude ~60: exp() of the raw score would overflow fp16/fp32 ranges without the running max
     _check(4, 64, 256, 64, 64, 4, scale=1.0, seed=5, tol=3e-2)
