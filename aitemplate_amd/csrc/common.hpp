@@ -93,17 +93,23 @@ AITAMD_DEVICE uint32_t clamp_records(int64_t bytes) {
 // Workgroup -> tile mapping.  The hardware deals consecutive workgroup ids
 // round-robin over the 8 XCDs; tiles that share an A row-panel or a B
 // column-panel should land on the same XCD so the panel is fetched into one
-// L2 only.  Step 1 gives every XCD a contiguous range of logical tile ids,
-// step 2 walks that range in groups of kGroupM tile-rows, column by column.
+// L2 only.  Step 1 gives every XCD a contiguous range of logical (batch, tile) ids,
+// step 2 walks the tiles of a batch in groups of kGroupM tile-rows, column by column.
 // ---------------------------------------------------------------------------
 template <int kGroupM>
-AITAMD_DEVICE void map_tile(int wg, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int total = tiles_m * tiles_n;
+AITAMD_DEVICE void map_tile(int wg, int tiles_m, int tiles_n, int batch, int& b, int& tm, int& tn) {
+  // wg runs over batch * tiles_m * tiles_n workgroups; logical ids are batch-major, so an XCD's
+  // contiguous id range is a run of whole batches (plus at most two partial ones at its ends):
+  // the tiles of one batch share its operands through one L2 and fill its output rows together.
+  const int per_batch = tiles_m * tiles_n;
+  const int total = per_batch * batch;
   const int xcd = wg % kNumXcd;
   const int local = wg / kNumXcd;
   const int q = total / kNumXcd;
   const int r = total % kNumXcd;
-  const int id = xcd * q + (xcd < r ? xcd : r) + local;
+  const int flat = xcd * q + (xcd < r ? xcd : r) + local;
+  b = flat / per_batch;
+  const int id = flat - b * per_batch;
   const int group_sz = kGroupM * tiles_n;
   const int g = id / group_sz;
   const int first_m = g * kGroupM;

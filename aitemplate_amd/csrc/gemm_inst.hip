@@ -84,12 +84,11 @@ hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
   p.tiles_n = (p.N + Tile::BN - 1) / Tile::BN;
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles <= 0 || p.batch <= 0) return hipSuccess;
-  if (tiles > 0x7fffffffll) return hipErrorInvalidValue;
-  dim3 grid((unsigned)tiles, (unsigned)(p.batch < 65535 ? p.batch : 65535), 1);
+  // one workgroup per (batch, tile) pair, or, for the persistent kernels, one per CU walking them
+  const int64_t total = tiles * p.batch;
+  if (total > 0x7fffffffll) return hipErrorInvalidValue;
+  dim3 grid((unsigned)total, 1, 1);
   if constexpr (IsPersistent<Tile>::value) {
-    // one workgroup per CU walks (tile, batch) pairs
-    const int64_t total = tiles * p.batch;
-    if (total > 0x7fffffffll) return hipErrorInvalidValue;
     const int cus = device_cus(dev);
     grid = dim3((unsigned)(total < cus ? total : cus), 1, 1);
   }

@@ -87,8 +87,8 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
   const int r32 = lane & 31;
   const int h = lane >> 5;
 
-  int tm, tn;
-  map_tile<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  int batch, tm, tn;
+  map_tile<8>(blockIdx.x, p.tiles_m, p.tiles_n, p.batch, batch, tm, tn);
   const int m0 = tm * BM;
   const int n0 = tn * BN;
   const int rows_a = (p.M - m0) < BM ? (p.M - m0) : BM;
@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
 
   const int k_tiles = (p.K + BK - 1) / BK;
 
-  for (int batch = blockIdx.y; batch < p.batch; batch += gridDim.y) {
+  {
     const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)batch * p.sa + (int64_t)m0 * p.lda;
     const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)batch * p.sb + (int64_t)n0 * p.ldb;
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ab, clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2));
@@ -272,8 +272,6 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
         }
       }
     }
-    // The next batch iteration overwrites LDS stage 0; every wave has passed the
-    // loop's final barrier after its last LDS read, so no extra barrier is needed.
   }
 }
 

@@ -155,8 +155,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
   const int fr = lane % MT;  // row of the MFMA operand / column of the transposed result
   const int fq = lane / MT;  // which 8-wide k chunk of the MFMA step this lane feeds
 
-  int tm, tn;
-  map_tile<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  int batch, tm, tn;
+  map_tile<8>(blockIdx.x, p.tiles_m, p.tiles_n, p.batch, batch, tm, tn);
   const int m0 = tm * BM;
   const int n0 = tn * BN;
   const int rows_a = (p.M - m0) < BM ? (p.M - m0) : BM;
@@ -189,7 +189,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
 
   const int k_tiles = (p.K + BK - 1) / BK;
 
-  for (int batch = blockIdx.y; batch < p.batch; batch += gridDim.y) {
+  {
     const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)batch * p.sa + (int64_t)m0 * p.lda;
     const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)batch * p.sb + (int64_t)n0 * p.ldb;
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ab, clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2));
@@ -397,8 +397,6 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
-    // all waves must be done with their strips before the next batch's slabs land
-    __syncthreads();
   }
 }
 

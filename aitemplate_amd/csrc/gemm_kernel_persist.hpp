@@ -109,11 +109,9 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   };
   auto tile_coord = [&](int i) {
     TileCoord c;
-    const int v = g + i * G;
-    const int b = v / tiles_per_batch;
-    const int t = v - b * tiles_per_batch;
-    int tm, tn;
-    map_tile<8>(t, p.tiles_m, p.tiles_n, tm, tn);
+    // virtual workgroup index: with one workgroup per CU, g % 8 is the XCD and stays it for every i
+    int b, tm, tn;
+    map_tile<8>(g + i * G, p.tiles_m, p.tiles_n, p.batch, b, tm, tn);
     c.m0 = tm * BM;
     c.n0 = tn * BN;
     c.batch = b;

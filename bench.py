@@ -80,6 +80,38 @@ def time_gemm(torch, eager, name, steps, warmup, algo=-1):
             "flops": 2 * M * N * K, "bytes": 2 * (M * K + N * K + N + (1 + nres) * M * N)}
 
 
+def time_call(torch, fn, steps, warmup):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def time_c4_c5(torch, eager, steps, warmup):
+    """bmm_rcr (config 4, against the HBM roofline) and bmm_softmax_bmm_permute (config 5)."""
+    g = torch.Generator(device="cuda").manual_seed(4)
+    sets4 = [(torch.randn(768, 384, 64, device="cuda", generator=g).half() / 8,
+              torch.randn(768, 384, 64, device="cuda", generator=g).half() / 8,
+              torch.empty(768, 384, 384, device="cuda", dtype=torch.float16)) for _ in range(3)]
+    ms4 = time_call(torch, lambda i: eager.bmm_rcr(sets4[i % 3][0], sets4[i % 3][1], out=sets4[i % 3][2]), steps, warmup)
+    b4 = 2 * 768 * (2 * 384 * 64 + 384 * 384)
+    sets5 = [tuple(torch.randn(16, 4096, 40, device="cuda", generator=g).half() for _ in range(3)) for _ in range(16)]
+    out5 = torch.empty(2, 4096, 8, 40, device="cuda", dtype=torch.float16)
+    ms5 = time_call(torch, lambda i: eager.bmm_softmax_bmm_permute(*sets5[i % 16], shape=(8,), scale=40 ** -0.5, out=out5),
+                    steps, warmup)
+    f5 = 4 * 16 * 4096 * 4096 * 40
+    return {"c4": {"op": "bmm_rcr", "ms": round(ms4, 5), "gbs": round(b4 / ms4 / 1e6, 1),
+                   "frac_of_hbm_peak": round(b4 / ms4 / 1e6 / PEAK_HBM_GBS, 4)},
+            "c5": {"op": "bmm_softmax_bmm_permute", "ms": round(ms5, 5), "tflops": round(f5 / ms5 / 1e9, 2),
+                   "frac_of_mfma_peak": round(f5 / ms5 / 1e9 / PEAK_FP16_TFLOPS, 4)}}
+
+
 def pick_instance(torch, eager, kernels, name, iters=15):
     """Untimed selection pass, the same procedure compile_model's profiling step applies
     (python/aitemplate/compiler/ops/gemm_universal/gemm_common.py:743-829 in the reference):
@@ -228,6 +260,7 @@ def main():
             t = o["event_ms_per_launch"] * 1e-3
             others[name] = {"op": SHAPES[name][0], "ms": round(o["event_ms_per_launch"], 5),
                             "tflops": round(o["flops"] / t / 1e12, 2), "gbs": round(o["bytes"] / t / 1e9, 1)}
+        others.update(time_c4_c5(torch, eager, max(20, args.steps // 4), max(5, args.warmup // 4)))
         line["other_configs"] = others
     if not args.no_in_abi:
         line["in_abi"] = in_abi(torch)
