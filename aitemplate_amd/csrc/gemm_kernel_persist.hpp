@@ -86,8 +86,18 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   const int total_tiles = tiles_per_batch * p.batch;
   const int G = gridDim.x;
   const int g = blockIdx.x;
-  const int my_tiles = (total_tiles - g + G - 1) / G;
   const int k_tiles = (p.K + BK - 1) / BK;
+  // Work items of this workgroup: one tile per full round, then its share of the last, partly
+  // filled round.  When at most half the workgroups would get a tile there, every leftover tile is
+  // split into an upper and a lower half (the waves of the other half idle through it): two
+  // workgroups finish a leftover tile in about half a tile time instead of one working while
+  // another waits.  Both halves of a tile go to workgroups of the same XCD.
+  const int full_rounds = total_tiles / G;
+  const int left = total_tiles - full_rounds * G;
+  const bool split = Tile::WGM == 2 && left > 0 && 2 * left <= G && (G % 16) == 0;
+  const int split_tile = ((g >> 4) << 3) + (g & 7);  // leftover tile of this workgroup when splitting
+  const int split_half = (g >> 3) & 1;
+  const int my_tiles = full_rounds + (split ? (split_tile < left ? 1 : 0) : (g < left ? 1 : 0));
 
   // ---- loader: a stream of slabs that runs across this workgroup's tiles ------------------------
   const int l_row = lane / Tile::CPR;
@@ -106,15 +116,18 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   struct TileCoord {
     int m0, n0, batch;
+    int rows;  // rows of the tile this workgroup computes: BM, or BM / 2 for half a leftover tile
   };
   auto tile_coord = [&](int i) {
     TileCoord c;
     // virtual workgroup index: with one workgroup per CU, g % 8 is the XCD and stays it for every i
     int b, tm, tn;
-    map_tile<8>(g + i * G, p.tiles_m, p.tiles_n, p.batch, b, tm, tn);
-    c.m0 = tm * BM;
+    const bool half = split && i == full_rounds;
+    map_tile<8>(half ? full_rounds * G + split_tile : g + i * G, p.tiles_m, p.tiles_n, p.batch, b, tm, tn);
+    c.m0 = tm * BM + (half ? split_half * (BM / 2) : 0);
     c.n0 = tn * BN;
     c.batch = b;
+    c.rows = half ? BM / 2 : BM;
     return c;
   };
 
@@ -123,11 +136,12 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   auto set_loader_tile = [&](int i) {
     if (i < my_tiles) {
       const TileCoord c = tile_coord(i);
-      const int rows_a = (p.M - c.m0) < BM ? (p.M - c.m0) : BM;
+      const int rows_a = (p.M - c.m0) < c.rows ? (p.M - c.m0) : c.rows;
       const int rows_b = (p.N - c.n0) < BN ? (p.N - c.n0) : BN;
       const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)c.batch * p.sa + (int64_t)c.m0 * p.lda;
       const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)c.batch * p.sb + (int64_t)c.n0 * p.ldb;
-      ra = make_rsrc(Ab, clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2));
+      // (the lower half of a leftover tile can lie wholly below M: nothing to fetch then)
+      ra = make_rsrc(Ab, rows_a > 0 ? clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2) : 0u);
       rb = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
     } else {
       // past the last tile the ring keeps turning on zero-sized buffers: every lane is out of
@@ -282,30 +296,40 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   for (int i = 0; i < my_tiles; ++i) {
     const TileCoord cur = tile_coord(i);
+    // waves whose rows lie outside a half tile keep the ring turning (their share of the loads, the
+    // waits and the barriers) but multiply and store nothing; a half tile is always the last item
+    const bool active = wm * Tile::WTM < cur.rows;
     for (int kt = 0; kt < k_tiles; ++kt) {
       const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
       const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
       const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
-      // first step: the rest of the slab whose first portion went out in the previous step
-      issue_part(L_P0, L);
-      load_frags(cur_st, 1, af[1], bf[1]);
-      if (kt == 0)
-        mfmas_first(af[0], bf[0]);
-      else
-        mfmas(af[0], bf[0]);
-      sched_step<MI * NI, MI + NI, L - L_P0>();
-      // last step: the next slab has landed once at most (NS-3) younger slabs are in flight; past
-      // the barrier nobody reads the previous slab any more, so its ring slot starts taking a new
-      // slab, and the next slab's first fragments are fetched under this slab's last MFMAs
-      wait_vmcnt<(NS - 3) * L>();
-      __builtin_amdgcn_s_barrier();
-      issue_part(0, L_P0);
-      load_frags(nxt_st, 0, af[0], bf[0]);
-      mfmas(af[1], bf[1]);
-      sched_step<MI * NI, MI + NI, L_P0>();
+      if (active) {
+        // first step: the rest of the slab whose first portion went out in the previous step
+        issue_part(L_P0, L);
+        load_frags(cur_st, 1, af[1], bf[1]);
+        if (kt == 0)
+          mfmas_first(af[0], bf[0]);
+        else
+          mfmas(af[0], bf[0]);
+        sched_step<MI * NI, MI + NI, L - L_P0>();
+        // last step: the next slab has landed once at most (NS-3) younger slabs are in flight; past
+        // the barrier nobody reads the previous slab any more, so its ring slot starts taking a new
+        // slab, and the next slab's first fragments are fetched under this slab's last MFMAs
+        wait_vmcnt<(NS - 3) * L>();
+        __builtin_amdgcn_s_barrier();
+        issue_part(0, L_P0);
+        load_frags(nxt_st, 0, af[0], bf[0]);
+        mfmas(af[1], bf[1]);
+        sched_step<MI * NI, MI + NI, L_P0>();
+      } else {
+        issue_part(L_P0, L);
+        wait_vmcnt<(NS - 3) * L>();
+        __builtin_amdgcn_s_barrier();
+        issue_part(0, L_P0);
+      }
       rd_stage = nx_stage;
     }
-    epilogue(cur);
+    if (active) epilogue(cur);
   }
   // no LDS-DMA may be in flight into a workgroup that has ended
   wait_vmcnt<0>();

@@ -66,6 +66,9 @@ def test_persist_instances_exist():
     (2048, 1536, 256),   # 48 tiles < CUs
     (8192, 3072, 768),   # 384 tiles: one or two per workgroup
     (12608, 1024, 96),   # unaligned M, three slabs
+    (4000, 4352, 64),    # 272 tiles on 256 CUs: the 16 leftover tiles are split in halves; M tail of 160 rows
+    (3900, 4352, 64),    # same, M tail of 60 rows: some lower halves lie wholly below M
+    (24576, 768, 128),   # 288 tiles: one full round plus 32 split tiles
 ])
 def test_persist_shapes(name, shape):
     M, N, K = shape
