@@ -29,6 +29,8 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE 95421.4 KiB x 2.000 (copy: 131084.6 read for 262144 KiB) + WRITE_SIZE 147456 KiB x 1.000
     "gemm_rcr_f16_256x256x32_w2x4_dma4_o1_p1_m32_c0": 346_412_000,
+    # FETCH_SIZE 97796.0 KiB x 2.000 + WRITE_SIZE 147456 KiB x 1.000
+    "gemm_rcr_f16_256x256x32_w2x4_persist4": 351_281_000,
 }
 
 SHAPES = {
