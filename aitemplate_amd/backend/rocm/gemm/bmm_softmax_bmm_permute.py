@@ -1,4 +1,4 @@
-"""Registry hooks of bmm_softmax_bmm_permute (and its causal variant).
+"""Registry hooks of bmm_softmax_bmm_permute, its causal variant and bmm_softmax_bmm.
 
 Replaces python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:32-388.  The launcher
 keeps the reference's shape: the 4th pointer is V, the dim pointers cover Q, K and the [B, M, O]
@@ -10,7 +10,8 @@ from ... import registry
 from ...target import Target
 from . import common
 
-_OPS = ("bmm_softmax_bmm_permute", "bmm_softmax_bmm_permute_causal")
+# bmm_softmax_bmm (reference hooks: backend/rocm/gemm/bmm_softmax_bmm.py) is the one-head case of the same launcher
+_OPS = ("bmm_softmax_bmm_permute", "bmm_softmax_bmm_permute_causal", "bmm_softmax_bmm")
 _INSTANCE = "attention_q128"
 
 

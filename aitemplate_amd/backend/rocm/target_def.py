@@ -38,6 +38,9 @@ class ROCM(Target):
     def arch(self) -> str:
         return self._arch
 
+    def device_name(self) -> str:
+        return f"rocm-{self._arch}"
+
     def cc(self) -> str:
         return os.environ.get("AIT_HOST_CXX", "g++")
 

@@ -20,7 +20,7 @@ from collections import OrderedDict
 from dataclasses import dataclass
 from enum import Enum
 from hashlib import sha1
-from typing import Any, Dict, List, Union
+from typing import Any, Dict, List, Optional, Union
 
 from ....backend import registry
 from ....backend.target import Target
@@ -85,6 +85,27 @@ def default_align_ab(a: int, b: int, dtype: str) -> int:
     return alignment.find_max_alignment(math.gcd(a, b), dtype)
 
 
+def profile_cache_args(func_attrs: Dict[str, Any], exec_key: str) -> Optional[Dict[str, Any]]:
+    """Key of one workload in the profiling-result cache (reference: the GemmQueryEntry built at
+    gemm_common.py:436-458), or None when no target is active."""
+    from ....backend import target as target_mod
+    from ....backend.profiler_cache import exec_entry_sha1
+
+    if target_mod.CURRENT_TARGET is None or "inputs" not in func_attrs or not func_attrs.get("op_instance"):
+        return None
+    names = sorted(func_attrs["op_instance"].keys())
+    shape = func_attrs.get("shape")
+    entry = exec_key if shape is None else f"{exec_key} | shape={tuple(shape)} | causal={func_attrs.get('causal')}"
+    return {
+        "op_type": func_attrs["op"],
+        "dtype": func_attrs["inputs"][0]._attrs["dtype"],
+        "device": target_mod.CURRENT_TARGET.device_name(),
+        "instances_sha1": sha1(";".join(names).encode("utf-8")).hexdigest(),
+        "exec_entry": entry,
+        "exec_entry_sha1": exec_entry_sha1(entry),
+    }
+
+
 class GemmProfilerPostprocessingDelegate:
     """Collects the profiler runs of all GEMM ops and, once they have finished, writes the
     fastest instance of each workload into the op's exec_path
@@ -114,6 +135,10 @@ class GemmProfilerPostprocessingDelegate:
             attrs["workspace"] = max(attrs["workspace"], res.workspace)
             attrs["split_k"] = split_k
             _LOGGER.info("Profiler (%s %s) selected %s: %.4f ms", attrs["op"], exec_key, name, res.duration)
+            args = profile_cache_args(attrs, exec_key)
+            if args is not None:
+                args.update(algo=name, workspace=res.workspace, split_k=split_k, duration=res.duration)
+                Target.current().insert_profile_cache("gemm", args)
 
 
 class gemm(Operator):
@@ -271,6 +296,15 @@ class gemm(Operator):
             if target.use_dummy_profiling_results() or profiler_runner is None:
                 item.algo = registry.get(self._registry_key("select_algo"))(self._attrs, key)
                 self._attrs["workspace"] = 0
+                continue
+            # a workload that was timed before (same op, type, device and instance list) is not timed again
+            args = profile_cache_args(self._attrs, key)
+            cached = None if args is None or target.force_profile() else target.query_profile_cache("gemm", args)
+            if cached is not None and cached[0] in self._attrs["op_instance"]:
+                _LOGGER.info("Load profiling result for %s %s from cache: %s", self._attrs["op"], key, cached)
+                item.algo = cached[0]
+                self._attrs["workspace"] = max(self._attrs["workspace"], cached[1])
+                self._attrs["split_k"] = cached[2]
                 continue
             cmd = self._gen_profile_cmd(prefix, filename, key)
             profiler_runner.push(cmd, process_result_callback=None, func_attrs=self._attrs,

@@ -172,6 +172,25 @@ def test_bmm_softmax_bmm_permute(bs, ms, N, K, D, heads, causal, copy_op):   # t
         torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("B,M,N,K,D,copy_op", [(24, 256, 256, 64, 64, False), (5, 100, 49, 40, 40, True)])
+def test_bmm_softmax_bmm(B, M, N, K, D, copy_op):   # the non-permuted op (reference: test_bmm_softmax_bmm.py:59-118)
+    X = Tensor(shape=[B, M, K], name="input_0", is_input=True)
+    B0 = Tensor(shape=[B, N, K], name="input_1", is_input=True)
+    B1 = Tensor(shape=[B, N, D], name="input_2", is_input=True)
+    scale = K ** -0.5
+    OP = ops.bmm_softmax_bmm(scale=scale)
+    if copy_op:
+        OP = ops.bmm_softmax_bmm(**OP._get_op_attributes())
+    Y = _mark_output(OP(X, B0, B1))
+    assert [d.value() for d in Y.shape()] == [B, M, D]
+    module = compile_model(Y, detect_target(), WORKDIR, f"attn_plain_{next(_counter)}")
+    q, k, v = _rand((B, M, K), 1), _rand((B, N, K), 2), _rand((B, N, D), 3)
+    want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, scale, 1).reshape(B, M, D).half().float()
+    y = torch.empty(B, M, D, dtype=torch.float16, device="cuda")
+    module.run_with_tensors([q.cuda(), k.cuda(), v.cuda()], [y])
+    torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
+
+
 # ---- the five benchmark configurations, full size, through the C ABI ----------------------
 @pytest.mark.parametrize("cfg", ["c1", "c2a", "c2b", "c3", "c4", "c5"])
 def test_benchmark_config_through_compile_model(cfg):

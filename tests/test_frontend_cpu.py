@@ -170,7 +170,7 @@ def test_registry_has_every_hook_for_every_op():
     detect_target()  # importing the ROCm backend registers the hooks
     for op in ("gemm_rcr", "gemm_rcr_bias", "gemm_rcr_bias_relu", "gemm_rcr_bias_gelu", "gemm_rcr_bias_fast_gelu",
                "gemm_rcr_bias_add", "gemm_rcr_bias_add_add", "bmm_rcr", "bmm_softmax_bmm_permute",
-               "bmm_softmax_bmm_permute_causal"):
+               "bmm_softmax_bmm_permute_causal", "bmm_softmax_bmm"):
         for hook in ("config", "filter", "gen_profiler", "gen_function", "func_decl", "func_call"):
             assert registry.exists(f"rocm.{op}.{hook}"), f"rocm.{op}.{hook}"
     with pytest.raises(RuntimeError):
@@ -340,3 +340,78 @@ def test_compile_model_builds_a_library_exporting_the_whole_abi(tmp_path, monkey
     # nothing else leaks out of the model library except the C ABI
     others = [l.split()[-1] for l in out.splitlines() if " T " in l and "AITemplate" not in l]
     assert not [s for s in others if not s.startswith("_")], others
+
+
+# ---- profiling-result cache -------------------------------------------------------------------
+def test_profile_cache_db_roundtrip(tmp_path):
+    from aitemplate_amd.backend.profiler_cache import ProfileCacheDB, exec_entry_sha1
+
+    db = ProfileCacheDB("rocm", path=str(tmp_path / "rocm.db"))
+    key = {"op_type": "gemm_rcr_bias", "dtype": "float16", "device": "rocm-gfx950", "instances_sha1": "abc",
+           "exec_entry": "M == 256 && N == 1024 && K == 1024",
+           "exec_entry_sha1": exec_entry_sha1("M == 256 && N == 1024 && K == 1024")}
+    assert db.query_gemm(key) is None
+    db.insert_gemm(dict(key, algo="tile_b", workspace=0, split_k=1, duration=0.25))
+    assert db.query_gemm(key) == ("tile_b", 0, 1)
+    db.insert_gemm(dict(key, algo="tile_c", workspace=0, split_k=1, duration=0.1))  # first writer wins
+    assert db.query_gemm(key) == ("tile_b", 0, 1) and db.num_entries() == 1
+    # any key component that differs is a miss: other instance list, other device, other workload
+    assert db.query_gemm(dict(key, instances_sha1="other")) is None
+    assert db.query_gemm(dict(key, device="rocm-gfx942")) is None
+    assert db.query_gemm(dict(key, exec_entry_sha1=exec_entry_sha1("M == 1 && N == 2 && K == 3"))) is None
+    with pytest.raises(KeyError):
+        db.query_gemm({"op_type": "gemm_rcr"})
+    db.close()
+    # persisted on disk
+    db2 = ProfileCacheDB("rocm", path=str(tmp_path / "rocm.db"))
+    assert db2.query_gemm(key) == ("tile_b", 0, 1)
+    db2.close()
+
+
+def test_profile_results_are_cached_and_reused(tmp_path, monkeypatch):
+    """Second profile() of the same workload takes the winner from the cache and runs no profiler
+    (reference flow: gemm_common.py:618-676); FORCE_PROFILE=1 times again; CI mode has no cache."""
+    from aitemplate_amd.compiler.ops.gemm_universal.gemm_common import GemmProfilerPostprocessingDelegate
+
+    monkeypatch.delenv("CI_FLAG", raising=False)
+    monkeypatch.setenv("CACHE_DIR", str(tmp_path / "cache"))
+    fake = tmp_path / "fake_profiler.sh"
+
+    def build_op():
+        op = list(_gemm_bias_graph(Ms=(4096,), N=64, K=64).src_ops())[0]
+        op.gen_profiler(str(tmp_path), DynamicProfileStrategy.MAX)
+        exe = os.path.join(str(tmp_path), "profiler", "gemm_rcr_bias", op._get_profiler_filename())
+        names = list(op._attrs["op_instance"])
+        os.remove(exe)
+        fake.write_text("#!/bin/sh\necho ran >> %s\n" % (tmp_path / "runs.log")
+                        + "".join(f"echo OP:{n},TIME:{1.0 + i},WS:0\n" for i, n in enumerate(names[:-1]))
+                        + f"echo OP:{names[-1]},TIME:0.5,WS:0\n")
+        fake.chmod(fake.stat().st_mode | stat.S_IEXEC)
+        os.symlink(str(fake), exe)
+        return op, names
+
+    def profile(op):
+        pr = ProfilerRunner(devices=["0"], postprocessing_delegate=GemmProfilerPostprocessingDelegate(), timeout=30)
+        op.profile(pr, str(tmp_path))
+        pr.join()
+
+    with detect_target() as target:
+        assert target.get_profile_cache_path() == str(tmp_path / "cache" / "rocm.db")
+        op, names = build_op()
+        profile(op)
+        key = list(op._attrs["exec_path"])[0]
+        assert op._attrs["exec_path"][key].algo == names[-1]
+        assert (tmp_path / "runs.log").read_text().count("ran") == 1
+    with detect_target():
+        op2, _ = build_op()
+        profile(op2)
+        assert op2._attrs["exec_path"][key].algo == names[-1]
+        assert (tmp_path / "runs.log").read_text().count("ran") == 1  # served from the cache
+        monkeypatch.setenv("FORCE_PROFILE", "1")
+        op3, _ = build_op()
+        profile(op3)
+        assert (tmp_path / "runs.log").read_text().count("ran") == 2
+        monkeypatch.delenv("FORCE_PROFILE")
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    with detect_target() as target:
+        assert target.get_profile_cache_path() is None
