@@ -10,10 +10,21 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 
-template <class T, int KS, int OT, bool VEC>
+// WIDE: eight waves (256 query rows) share each K / V tile and four LDS stages keep three tiles in
+// flight; otherwise four waves, two stages and two workgroups per CU.
+template <int KS, int OT, bool WIDE>
+struct TileOf {
+  using type = AttnTile<KS, OT>;
+};
+template <int KS, int OT>
+struct TileOf<KS, OT, true> {
+  using type = AttnTile<KS, OT, ((16 * KS + 32 * OT) <= 128 ? 128 : 64), 8, 4>;
+};
+
+template <class T, int KS, int OT, bool VEC, bool DMA, bool WIDE>
 hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
-  using Tile = AttnTile<KS, OT>;
-  auto kernel = attention_kernel<T, Tile, VEC>;
+  using Tile = typename TileOf<KS, OT, WIDE>::type;
+  auto kernel = attention_kernel<T, Tile, VEC, DMA>;
   static std::once_flag once[kMaxDevices];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -32,10 +43,10 @@ hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
 
 typedef hipError_t (*AttnLaunch)(const AttnParams&, hipStream_t);
 
-template <class T, bool VEC>
+template <class T, bool VEC, bool DMA, bool WIDE>
 AttnLaunch pick(int ks, int ot) {
 #define AITAMD_ATTN_CASE(KS, OT) \
-  if (ks <= KS && ot <= OT) return &launch_attention<T, KS, OT, VEC>;
+  if (ks <= KS && ot <= OT) return &launch_attention<T, KS, OT, VEC, DMA, WIDE>;
   // smallest padded head dims first; (K <= 16 KS, O <= 32 OT)
   AITAMD_ATTN_CASE(2, 1)
   AITAMD_ATTN_CASE(3, 2)
@@ -88,11 +99,22 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
   const int ot = (int)((O + 31) / 32);
   const bool vec = (K % 8 == 0) && (O % 8 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15) == 0) &&
       ((reinterpret_cast<uintptr_t>(k) & 15) == 0) && ((reinterpret_cast<uintptr_t>(v) & 15) == 0);
+  // direct-to-LDS tiles address K and V of one batch entry with 32-bit byte offsets
+  const int64_t kv_dim = K > O ? K : O;
+  // (tiles are issued up to three past the last one, hence the slack)
+  const bool dma = vec && (N + 4 * 128) * kv_dim * 2 < 0x7fffffffll;
+  // 256-row workgroups for small head dims (where re-streaming K / V per 128 query rows costs most; measured
+  // slower at head dims 64 and 128) once there are enough of them to fill the CUs
+  const bool wide = dma && (16 * ks + 32 * ot) <= 112 && ((M + 255) / 256) * B >= 256;
   AttnLaunch fn = nullptr;
   if (dtype == 0)
-    fn = vec ? pick<f16, true>(ks, ot) : pick<f16, false>(ks, ot);
+    fn = wide ? pick<f16, true, true, true>(ks, ot)
+              : (dma ? pick<f16, true, true, false>(ks, ot)
+                     : (vec ? pick<f16, true, false, false>(ks, ot) : pick<f16, false, false, false>(ks, ot)));
   else
-    fn = vec ? pick<bf16, true>(ks, ot) : pick<bf16, false>(ks, ot);
+    fn = wide ? pick<bf16, true, true, true>(ks, ot)
+              : (dma ? pick<bf16, true, true, false>(ks, ot)
+                     : (vec ? pick<bf16, true, false, false>(ks, ot) : pick<bf16, false, false, false>(ks, ot)));
   if (!fn) return fail("aitamd_bmm_softmax_bmm_permute: no instance for K=%lld O=%lld", (long long)K, (long long)O);
   const hipError_t e = fn(p, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail("aitamd_bmm_softmax_bmm_permute: launch failed: %s", hipGetErrorString(e));

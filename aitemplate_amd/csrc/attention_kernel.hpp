@@ -37,22 +37,26 @@ struct AttnParams {
   int32_t causal;
 };
 
-template <int KS_, int OT_, int BN_ = ((16 * KS_ + 32 * OT_) <= 112 ? 128 : 64)>
+// NW_ waves (32 query rows each) share the K / V tiles; NS_ LDS stages.  The register-staged
+// loaders use two stages; the direct-to-LDS path keeps NS_ - 1 tiles in flight.
+template <int KS_, int OT_, int BN_ = ((16 * KS_ + 32 * OT_) <= 112 ? 128 : 64), int NW_ = 4, int NS_ = 2>
 struct AttnTile {
   static constexpr int KS = KS_;          // K padded to 16 * KS
   static constexpr int OT = OT_;          // O padded to 32 * OT
   static constexpr int KP = 16 * KS;
   static constexpr int OP = 32 * OT;
-  static constexpr int BM = 128;          // query rows per workgroup (4 waves x 32)
+  static constexpr int NW = NW_, NS = NS_;
+  static constexpr int BM = 32 * NW;      // query rows per workgroup
   static constexpr int BN = BN_;          // keys per LDS tile: 128 while two workgroups still fit one CU's LDS
-  static constexpr int NT = 256;
+  static constexpr int NT = 64 * NW;
   static constexpr int K_PITCH = KP + 8;  // halves; keeps 16 consecutive rows on distinct banks
   static constexpr int V_PITCH = OP + 8;
   static constexpr int K_CHUNKS = BN * KP / 8;  // 16-byte chunks per tile (pads included)
   static constexpr int V_CHUNKS = BN * OP / 8;
   static constexpr int K_IT = (K_CHUNKS + NT - 1) / NT;
   static constexpr int V_IT = (V_CHUNKS + NT - 1) / NT;
-  static constexpr int kLdsBytes = 2 * BN * (K_PITCH + V_PITCH) * 2;
+  static constexpr int kLdsBytes = NS * BN * (K_PITCH + V_PITCH) * 2;
+  static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
 };
 
 // LDS transpose read: 4 x 16-bit per lane, gathered across the 16 lanes of a block
@@ -91,8 +95,35 @@ AITAMD_DEVICE float sum_across_halves(float x) {
 
 // VEC: K and O are multiples of 8 and all base pointers 16-byte aligned -> 128-bit
 // loads; otherwise elements are gathered one by one (slow, any shape).
-template <class T, class Tile, bool VEC>
-__global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams p) {
+// DMA (needs VEC, and each K / V matrix of a batch entry below 2 GiB): the K / V tiles go
+// global -> LDS directly (buffer_load ... lds) instead of through registers: lane i of a wave-load
+// fills the i-th 16-byte chunk of a 1 KiB LDS block, the rows' pad chunk and the rows past N are
+// out-of-range lanes (zero fill), and one s_waitcnt vmcnt(0) + s_barrier per tile replaces the
+// register staging, the LDS stores and the full __syncthreads().
+template <int N>
+AITAMD_DEVICE void attn_wait_vmcnt() {
+  // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]; only vmcnt is waited for
+  constexpr int imm = (N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8);
+  __builtin_amdgcn_s_waitcnt(imm);
+}
+template <int N>
+AITAMD_DEVICE void attn_wait_vmcnt_upto(int n) {
+  // wave-uniform n: waits until at most min(n, N) vector-memory operations are outstanding
+  if constexpr (N == 0) {
+    attn_wait_vmcnt<0>();
+  } else {
+    if (n >= N)
+      attn_wait_vmcnt<N>();
+    else
+      attn_wait_vmcnt_upto<N - 1>(n);
+  }
+}
+
+template <class T, class Tile, bool VEC, bool DMA = false>
+__global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_kernel(const AttnParams p) {
+  static_assert(!DMA || VEC, "the direct-to-LDS path needs 16-byte chunks");
+  static_assert(DMA || Tile::NS == 2, "the register-staged loaders double-buffer");
+  constexpr int NS = Tile::NS, NW = Tile::NW;
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
   using vec4 = typename Tr::vec4;
@@ -100,8 +131,8 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
   constexpr int BN = Tile::BN, KPI = Tile::K_PITCH, VPI = Tile::V_PITCH;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* const sK = reinterpret_cast<T*>(smem_raw);  // [2][BN][K_PITCH]
-  T* const sV = sK + 2 * BN * KPI;               // [2][BN][V_PITCH]
+  T* const sK = reinterpret_cast<T*>(smem_raw);  // [NS][BN][K_PITCH]
+  T* const sV = sK + NS * BN * KPI;              // [NS][BN][V_PITCH]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -184,6 +215,47 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
       }
     };
 
+    // ---- direct-to-LDS tile loader: the KL + VL wave-loads of a tile are dealt round-robin to the waves
+    constexpr int KC1 = KP / 8 + 1, VC1 = OP / 8 + 1;        // chunks per LDS row, pad chunk included
+    constexpr int KL = BN * KC1 / 64, VL = BN * VC1 / 64;     // wave-loads per K / V tile
+    constexpr int L_W = (KL + VL + NW - 1) / NW;
+    static_assert((BN * KC1) % 64 == 0 && (BN * VC1) % 64 == 0, "tiles must be whole wave-loads");
+    static_assert(Tile::K_PITCH == KC1 * 8 && Tile::V_PITCH == VC1 * 8, "LDS rows are the chunks of a row plus one");
+    typedef __attribute__((address_space(3))) void lds_void;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    uint32_t d_off[L_W];  // byte offset of the lane's chunk inside K (or V) for n0 = 0; kOobOffset = always zero
+    __amdgpu_buffer_rsrc_t rk, rv;
+    if constexpr (DMA) {
+#pragma unroll
+      for (int i = 0; i < L_W; ++i) {
+        const int j = wave_u + NW * i;
+        const bool is_k = j < KL;
+        const int idx = (is_k ? j : j - KL) * 64 + lane;
+        const int c1 = is_k ? KC1 : VC1;
+        const int dim = is_k ? p.K : p.O;
+        const int row = idx / c1, c = idx - row * c1;
+        d_off[i] = (c * 8 < dim) ? (uint32_t)((row * dim + c * 8) * 2) : kOobOffset;
+      }
+      rk = make_rsrc(Kb, (uint32_t)((int64_t)p.N * p.K * 2));
+      rv = make_rsrc(Vb, (uint32_t)((int64_t)p.N * p.O * 2));
+    }
+    auto issue_tile = [&](int n0, int stage) {
+      T* dK = sK + stage * BN * KPI;
+      T* dV = sV + stage * BN * VPI;
+#pragma unroll
+      for (int i = 0; i < L_W; ++i) {
+        const int j = wave_u + NW * i;
+        if (j >= KL + VL) continue;
+        if (j < KL) {
+          const uint32_t off = d_off[i] != kOobOffset ? d_off[i] + (uint32_t)(n0 * p.K * 2) : kOobOffset;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_void*)(dK + j * 512), 16, off, 0, 0, 0);
+        } else {
+          const uint32_t off = d_off[i] != kOobOffset ? d_off[i] + (uint32_t)(n0 * p.O * 2) : kOobOffset;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_void*)(dV + (j - KL) * 512), 16, off, 0, 0, 0);
+        }
+      }
+    };
+
     // keys this workgroup has to visit (causal: nothing right of the last query row)
     int n_end = p.N;
     if (p.causal) {
@@ -204,11 +276,22 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
     float m_run = m_init;
     float l_run = 0.0f;       // running sum over this lane's half of the keys
 
-    if (n_tiles > 0) {
-      load_tiles(0);
-      store_tiles(0);
+    // wave-loads this wave issues per tile
+    const int my_loads = (KL + VL - wave_u + NW - 1) / NW;
+    if constexpr (DMA) {
+      // NS - 1 tiles in flight; tiles past the last one are all out of range (zero fill, no traffic),
+      // issued all the same so that the number of loads per tile stays constant for the waits
+      if (n_tiles > 0) {
+#pragma unroll
+        for (int s0 = 0; s0 < NS - 1; ++s0) issue_tile(s0 * BN, s0);
+      }
+    } else {
+      if (n_tiles > 0) {
+        load_tiles(0);
+        store_tiles(0);
+      }
+      __syncthreads();
     }
-    __syncthreads();
 
     // source-lane address pattern of the LDS transpose read (see file header):
     // 16-lane block = one 4-key x 16-column patch; lane i of the block points at
@@ -217,10 +300,19 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
     const int tr_row = tr_i >> 2;
     const int tr_col = ((lane >> 4) & 1) * 16 + (tr_i & 3) * 4;
 
+    int cur = 0;
     for (int t = 0; t < n_tiles; ++t) {
-      const int cur = t & 1;
       const bool has_next = (t + 1) < n_tiles;
-      if (has_next) load_tiles((t + 1) * BN);
+      if constexpr (DMA) {
+        // this wave's part of tile t has landed once only the NS - 2 younger tiles are in flight; past
+        // the barrier everybody's has, and nobody reads the stage of tile t - 1 any more, so tile
+        // t + NS - 1 starts landing there
+        attn_wait_vmcnt_upto<(NS - 2) * L_W>((NS - 2) * my_loads);
+        __builtin_amdgcn_s_barrier();
+        issue_tile((t + NS - 1) * BN, cur == 0 ? NS - 1 : cur - 1);
+      } else {
+        if (has_next) load_tiles((t + 1) * BN);
+      }
       const T* cK = sK + cur * BN * KPI;
       const T* cV = sV + cur * BN * VPI;
 
@@ -317,8 +409,11 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
         }
       }
 
-      if (has_next) store_tiles(cur ^ 1);
-      __syncthreads();
+      if constexpr (!DMA) {
+        if (has_next) store_tiles(cur ^ 1);
+        __syncthreads();
+      }
+      cur = cur + 1 == NS ? 0 : cur + 1;
     }
 
     // ---- normalise and store permuted: out[b / G][m][b % G][o]
@@ -345,6 +440,7 @@ __global__ void __launch_bounds__(Tile::NT, 2) attention_kernel(const AttnParams
           }
         }
     }
+    if constexpr (DMA) attn_wait_vmcnt<0>();  // the zero-fill tiles issued past the last one
     __syncthreads();  // LDS stage 0 is refilled by the next batch iteration
   }
 }
