@@ -46,6 +46,17 @@ NUM_RESIDUALS_OF_EPILOGUE = {0: 0, 1: 0, 2: 0, 3: 0, 4: 1, 5: 2, 6: 1, 7: 2, 8: 
                              10: 0, 11: 0, 12: 1, 13: 2, 14: 1, 15: 1, 16: 1}
 DTYPE_ID = {"float16": 0, "bfloat16": 1}
 
+# Ops that store through a 5-D output permutation: name -> (epilogue id, layout id of aitamd_gemm_rcr_permute).
+# On ROCm the reference lowers layout "20314" like "m3n2" (gemm_rcr_bias_permute.py:66-72 of
+# python/aitemplate/compiler/ops/gemm_universal/).
+PERMUTE_M2N3, PERMUTE_M3N2 = 1, 2
+PERMUTE_OPS = {
+    "gemm_rcr_permute_m2n3": (0, PERMUTE_M2N3),
+    "gemm_rcr_bias_permute_m2n3": (1, PERMUTE_M2N3),
+    "gemm_rcr_bias_permute_m3n2": (1, PERMUTE_M3N2),
+    "gemm_rcr_bias_permute": (1, PERMUTE_M3N2),
+}
+
 # Every symbol include/aitemplate_amd_kernels.h declares.
 EXPORTED_SYMBOLS = [
     "aitamd_version",
@@ -56,6 +67,7 @@ EXPORTED_SYMBOLS = [
     "aitamd_gemm_algo_supported",
     "aitamd_gemm_heuristic_algo",
     "aitamd_gemm_rcr",
+    "aitamd_gemm_rcr_permute",
     "aitamd_bmm_rcr",
     "aitamd_bmm_softmax_bmm_permute",
 ]
@@ -97,6 +109,8 @@ def load() -> ctypes.CDLL:
         lib.aitamd_gemm_heuristic_algo.argtypes = [i32, i32, i64, i64, i64, i64, i64, i64, i32]
         lib.aitamd_gemm_rcr.restype = i32
         lib.aitamd_gemm_rcr.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]
+        lib.aitamd_gemm_rcr_permute.restype = i32
+        lib.aitamd_gemm_rcr_permute.argtypes = [i32, i32, i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, i64, i64, i64, vp]
         lib.aitamd_bmm_rcr.restype = i32
         lib.aitamd_bmm_rcr.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
         lib.aitamd_bmm_softmax_bmm_permute.restype = i32

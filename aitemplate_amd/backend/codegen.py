@@ -17,7 +17,7 @@ from typing import Dict, List, Tuple
 
 from ..compiler.base import IntImm, Tensor
 from ..compiler.dtype import dtype_to_enumerator, get_dtype_size
-from ..compiler.transform.mark_param_tensor import storage_root
+from ..compiler.transform.mark_param_tensor import storage_offset_bytes, storage_root
 from ..compiler.transform.transform_utils import get_sorted_ops, is_view_op
 from . import registry
 from .target import Target
@@ -164,13 +164,17 @@ class ModelSource:
             else:
                 nbytes = f"({_numel_expr(t)}) * {get_dtype_size(t.dtype())}"
                 copies.append(
-                    f"    if (params_[{idx}].ptr != nullptr && params_[{idx}].ptr != {owner._attrs['name']})\n"
-                    f"      AIT_DEVICE_CHECK(hipMemcpyAsync(params_[{idx}].ptr, {owner._attrs['name']}, {nbytes}, "
+                    f"    if (params_[{idx}].ptr != nullptr && params_[{idx}].ptr != {n})\n"
+                    f"      AIT_DEVICE_CHECK(hipMemcpyAsync(params_[{idx}].ptr, {n}, {nbytes}, "
                     f"hipMemcpyDeviceToDevice, stream));")
         for t in self.graph:
             owner = t._attrs["external_tensor"]
             if owner is not None and not t.is_a_const_num():
-                lines.append(f"    {t._attrs['name']} = {owner._attrs['name']};")
+                rel = storage_offset_bytes(t) - storage_offset_bytes(owner)
+                if rel == 0:
+                    lines.append(f"    {t._attrs['name']} = {owner._attrs['name']};")
+                else:  # a piece of a split: same buffer, shifted
+                    lines.append(f"    {t._attrs['name']} = static_cast<uint8_t*>({owner._attrs['name']}) + ({rel});")
         return "\n".join(lines), "\n".join(copies)
 
     def meta(self) -> str:

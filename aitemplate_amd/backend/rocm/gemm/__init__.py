@@ -1,2 +1,2 @@
 """Importing this package registers the ROCm hooks of the GEMM family."""
-from . import bmm_rcr, bmm_softmax_bmm_permute, gemm_rcr_family  # noqa: F401
+from . import bmm_rcr, bmm_softmax_bmm_permute, gemm_rcr_family, gemm_rcr_permute  # noqa: F401

@@ -34,6 +34,8 @@ EXTRA_PTRS = {0: [], 1: ["bias_ptr"]}
 
 
 def epilogue_id(op_name: str) -> int:
+    if op_name in _kernels.PERMUTE_OPS:
+        return _kernels.PERMUTE_OPS[op_name][0]
     return _kernels.EPILOGUE_OF_OP[op_name]
 
 
@@ -184,11 +186,14 @@ namespace ait {
 FOOTER = "\n}  // namespace ait\n"
 
 
-def gemm_signature(func_name: str, op_name: str, a_rank: int, b_rank: int, c_rank: int) -> str:
+def gemm_signature(func_name: str, op_name: str, a_rank: int, b_rank: int, c_rank: int, pdims: int = 0) -> str:
+    """Launcher prototype; `pdims` trailing `const int p_dim<i>` carry a permuting op's shape attribute
+    (reference: backend/rocm/gemm/common.py:140-160)."""
     ptrs = ["void* in_ptr", "void* weight_ptr", "void* out_ptr"] + [f"void* {p}" for p in extra_pointer_names(op_name)]
     dims = [f"int64_t* {n}" for n in dim_param_names("a", a_rank) + dim_param_names("b", b_rank)
             + dim_param_names("c", c_rank)]
-    return f"void {func_name}({', '.join(ptrs + dims + ['hipStream_t stream'])})"
+    perm = [f"const int p_dim{i}" for i in range(pdims)]
+    return f"void {func_name}({', '.join(ptrs + dims + perm + ['hipStream_t stream'])})"
 
 
 def gemm_gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_dict) -> str:

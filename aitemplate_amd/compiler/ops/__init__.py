@@ -1,2 +1,2 @@
-from .common.view_ops import flatten, reshape  # noqa: F401
+from .common.view_ops import flatten, reshape, split  # noqa: F401
 from .gemm_universal import *  # noqa: F401,F403

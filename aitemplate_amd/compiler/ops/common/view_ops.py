@@ -1,10 +1,13 @@
-"""View ops: reshape (and flatten via reshape) — outputs alias their input's memory.
+"""View ops: reshape (and flatten via reshape) and split along the outermost dim — outputs alias their
+input's memory.
 
 Counterpart of the reshape in python/aitemplate/compiler/ops/common/view_ops.py, reduced
-to static target shapes with at most one -1 (what the GEMM-family graphs use)."""
-from typing import List, Union
+to static target shapes with at most one -1 (what the GEMM-family graphs use), and of
+python/aitemplate/compiler/ops/tensor/split.py:31-170 for the case that needs no copy."""
+from typing import List, Sequence, Union
 
 from ...base import IntImm, IntVar, Operator, Tensor
+from ...dtype import get_dtype_size
 
 
 class _view(Operator):
@@ -84,3 +87,70 @@ class flatten(reshape):
 
     def _get_op_attributes(self):
         return {"start_dim": self._attrs["start"], "end_dim": self._attrs["end"]}
+
+
+class split(_view):
+    """torch.split(x, split_size_or_sections, dim) -> tuple of tensors.
+
+    Only splits that leave every piece contiguous are supported (dim 0, or a dim preceded by dims of
+    size 1) with static shapes: each piece is then a view at a byte offset into x and no kernel runs.
+    This is the split nn.MultiheadAttention applies to the packed [3, batch, heads, seq, head_dim]
+    projection.  The reference materialises every split with a copy kernel unless a later pass removes
+    it (split.py:172-214)."""
+
+    def __init__(self):
+        super().__init__()
+        self._attrs["op"] = "split"
+        self._attrs["is_view_op"] = True
+        self._attrs["has_profiler"] = False
+
+    def __call__(self, x: Tensor, split_size_or_sections: Union[int, Sequence[int]], dim: int = 0):
+        shape = x._attrs["shape"]
+        rank = len(shape)
+        if rank <= 0:
+            raise RuntimeError("expected a non-scalar tensor")
+        if not -rank <= dim < rank:
+            raise RuntimeError(f"split dim ({dim}) expected to be less than rank ({rank})")
+        dim %= rank
+        if not all(isinstance(d, IntImm) for d in shape):
+            raise NotImplementedError("split needs static shapes on this backend")
+        if any(d.value() != 1 for d in shape[:dim]):
+            raise NotImplementedError("split along an inner dim would need a copy kernel; only dim 0 "
+                                      "(or a dim behind dims of size 1) is supported")
+        size = shape[dim].value()
+        if isinstance(split_size_or_sections, (list, tuple)):
+            sizes = [int(v.value()) if isinstance(v, IntImm) else int(v) for v in split_size_or_sections]
+            if len(sizes) < 1:
+                raise RuntimeError(f"the number of splits expected >=0 but got {len(sizes)}")
+            if sum(sizes) != size:
+                raise RuntimeError(f"sum of split_sizes ({sizes}) does not match split_dim_size ({size})")
+        else:
+            step = split_size_or_sections.value() if isinstance(split_size_or_sections, IntImm) \
+                else split_size_or_sections
+            if not isinstance(step, int):
+                raise RuntimeError("split_size expected to be of int")
+            if size == 0:
+                sizes = [0]
+            else:
+                if step <= 0:
+                    raise RuntimeError("split_size expected to be > 0")
+                sizes = [step] * (size // step) + ([size % step] if size % step else [])
+        self._attrs["inputs"] = [x]
+        self._attrs["split_dim"] = dim
+        self._attrs["split_sizes"] = sizes
+        self._set_depth()
+        inner = get_dtype_size(x.dtype())
+        for d in shape[dim + 1:]:
+            inner *= d.value()
+        outputs, start = [], 0
+        for n in sizes:
+            out_shape = list(shape[:dim]) + [IntImm(n)] + list(shape[dim + 1:])
+            t = Tensor(out_shape, src_ops={self}, is_view_of=x, dtype=x.dtype())
+            t._attrs["view_offset_bytes"] = start * inner
+            outputs.append(t)
+            start += n
+        self._attrs["outputs"] = outputs
+        return tuple(outputs)
+
+    def _get_op_attributes(self):
+        return {}

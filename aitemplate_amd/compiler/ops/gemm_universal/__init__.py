@@ -25,3 +25,4 @@ from .gemm_rcr_bias_broadcast import (  # noqa: F401
     gemm_rcr_bias_sigmoid_mul,
     gemm_rcr_bias_sigmoid_mul_tanh,
 )
+from .gemm_rcr_permute import gemm_rcr_bias_permute, gemm_rcr_permute  # noqa: F401

@@ -17,11 +17,22 @@ def storage_root(t: Tensor) -> Tensor:
     return t
 
 
+def storage_offset_bytes(t: Tensor) -> int:
+    """Byte offset of `t` inside its storage root (non-zero below a split view)."""
+    off = 0
+    while t._attrs["is_view_of"] is not None:
+        off += int(t._attrs.get("view_offset_bytes", 0) or 0)
+        t = t._attrs["is_view_of"]
+    return off
+
+
 def mark_param_tensor(sorted_graph: List[Tensor], output_tensors: List[Tensor] = None) -> None:
     """Sets is_param, and for every tensor that does not own its memory
     `external_tensor` = the tensor whose buffer it uses:
       * views of an input / constant use that parameter's memory,
-      * a group containing graph outputs lives in its first output's buffer,
+      * a group containing graph outputs lives in its first output's buffer, unless that output covers
+        only a part of the group's memory (it sits below a split): then the group keeps its own buffer
+        and the outputs are copied out after the ops ran,
       * otherwise views use the memory-planned buffer of the tensor they view."""
     for t in sorted_graph:
         if not t.src_ops():
@@ -33,7 +44,8 @@ def mark_param_tensor(sorted_graph: List[Tensor], output_tensors: List[Tensor] =
     for members in groups.values():
         root = storage_root(members[0])
         outs = sorted((m for m in members if m._attrs["is_output"]), key=lambda m: order.get(id(m), 1 << 30))
-        if root._attrs["is_param"] or not outs:
+        partial = any(storage_offset_bytes(m) != 0 or m.size_bytes() != root.size_bytes() for m in members)
+        if root._attrs["is_param"] or not outs or partial:
             owner = root
         else:
             owner = outs[0]

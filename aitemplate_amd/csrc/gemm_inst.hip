@@ -30,19 +30,22 @@ constexpr int kMaxDevices = 64;
 
 using Epi = Epilogue<AITAMD_EPI>;
 
-template <class Tile>
+// Kernels with the permuted store exist for the two epilogues the permuting ops use.
+constexpr bool kHasPermutedStore = AITAMD_EPI == kEpiNone || AITAMD_EPI == kEpiBias;
+
+template <class Tile, bool PERM>
 struct KernelOf {
-  static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi>;
+  static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi, PERM>;
 };
-template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
-struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, bool PERM>
+struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, PERM> {
   static constexpr auto value =
-      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, Epi>;
+      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, Epi, PERM>;
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int NS>
-struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS>> {
-  static constexpr auto value = gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS>, Epi>;
+template <int BM, int BN, int BK, int WM, int WN, int NS, bool PERM>
+struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS>, PERM> {
+  static constexpr auto value = gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS>, Epi, PERM>;
 };
 template <class Tile>
 struct IsPersistent {
@@ -64,9 +67,9 @@ inline int device_cus(int dev) {
   return v;
 }
 
-template <class Tile>
-hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
-  auto kernel = KernelOf<Tile>::value;
+template <class Tile, bool PERM>
+hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
+  auto kernel = KernelOf<Tile, PERM>::value;
   // LDS above 64 KiB has to be opted into once per device.
   static std::once_flag once[kMaxDevices];
   int dev = 0;
@@ -94,6 +97,15 @@ hipError_t launch_tile(const GemmParams& p_in, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kernel, grid, dim3(Tile::NT), Tile::kLdsBytes, stream, p);
   return hipGetLastError();
+}
+
+template <class Tile>
+hipError_t launch_tile(const GemmParams& p, hipStream_t stream) {
+  if (p.perm_on) {
+    if constexpr (kHasPermutedStore) return launch_kernel<Tile, true>(p, stream);
+    return hipErrorInvalidValue;
+  }
+  return launch_kernel<Tile, false>(p, stream);
 }
 
 // Workgroups one CU can hold: limited by LDS (160 KiB) and by the register file

@@ -34,7 +34,31 @@ struct GemmParams {
   int64_t lda, ldb, ldc, ldd;  // row pitches, in elements
   int64_t sa, sb, sc, sd;      // batch strides, in elements (0 broadcasts)
   int32_t tiles_m, tiles_n;
+  // Permuted store (kernels built with PERM; perm_on tells the launcher to pick them).  The row index splits as
+  // m = (m0 * perm_m1 + m1) * perm_m2 + m2 and the column index as n = (n0 * perm_n1 + n1) * perm_n2 + n2,
+  // and C[m, n] goes to element m0*sm0 + m1*sm1 + m2*sm2 + n0*sn0 + n1*sn1 + n2 of a contiguous buffer.
+  // That covers the reference's 5-D output permutations
+  // (python/aitemplate/backend/rocm/gemm/permute_common.py:20-130): "m2n3" has perm_m2 = 1, "m3n2" perm_n1 = 1.
+  int32_t perm_on, perm_m1, perm_m2, perm_n1, perm_n2;
+  int64_t perm_sm0, perm_sm1, perm_sm2, perm_sn0, perm_sn1;
 };
+
+// Element index of C[m, n] in the output buffer.  PERM is a template flag rather than a run-time test so
+// that the plain kernels carry none of the index arithmetic (in the large tiles the extra live values
+// cost registers the main loop needs).  The row and the column parts are separate so that a lane that
+// keeps one of them fixed across stores evaluates it once.
+template <bool PERM>
+AITAMD_DEVICE int64_t out_index(const GemmParams& p, int m, int n) {
+  if constexpr (!PERM) {
+    return (int64_t)m * p.ldc + n;
+  } else {
+    const int m01 = m / p.perm_m2, m2 = m - m01 * p.perm_m2;
+    const int m0 = m01 / p.perm_m1, m1 = m01 - m0 * p.perm_m1;
+    const int n01 = n / p.perm_n2, n2 = n - n01 * p.perm_n2;
+    const int n0 = n01 / p.perm_n1, n1 = n01 - n0 * p.perm_n1;
+    return (m0 * p.perm_sm0 + m1 * p.perm_sm1 + m2 * p.perm_sm2) + (n0 * p.perm_sn0 + n1 * p.perm_sn1 + n2);
+  }
+}
 
 // KVEC = number of K-contiguous elements that may be fetched with one load:
 // 8 -> 128-bit loads (K % 8 == 0, 16-byte aligned rows), 4/2/1 -> narrower
@@ -66,7 +90,7 @@ AITAMD_DEVICE int lds_chunk_elem(int row, int chunk) {
   return row * Tile::BK + ((chunk ^ swz) << 3);
 }
 
-template <class T, class Tile, class Epi>
+template <class T, class Tile, class Epi, bool PERM = false>
 __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) {
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
@@ -223,7 +247,7 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;
     const T* bias = reinterpret_cast<const T*>(p.bias);
 
-    bool vec_ok = ((p.N & 3) == 0) && ((p.ldc & 3) == 0) && ((p.sc & 3) == 0) &&
+    bool vec_ok = ((p.N & 3) == 0) && ((p.ldc & 3) == 0) && ((p.sc & 3) == 0) && (!PERM || (p.perm_n2 & 3) == 0) &&
         ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
     if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 7) == 0);
     if (Epi::kNumD >= 1)
@@ -244,7 +268,7 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
           float v[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) v[j] = acc[mi][ni][g * 4 + j];
-          const int64_t c_idx = (int64_t)m * p.ldc + n;
+          const int64_t c_idx = out_index<PERM>(p, m, n);
           const int64_t d_idx = (int64_t)m * p.ldd + n;
           if (vec_ok) {
             vec4 bv = {}, d0v = {}, d1v = {};
@@ -265,7 +289,7 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
                 if constexpr (Epi::kHasBias) bj = Tr::to_float(bias[n + j]);
                 if constexpr (Epi::kNumD >= 1) d0j = Tr::to_float(D0b[d_idx + j]);
                 if constexpr (Epi::kNumD >= 2) d1j = Tr::to_float(D1b[d_idx + j]);
-                Cb[c_idx + j] = Tr::from_float(Epi::apply(v[j], bj, d0j, d1j));
+                Cb[out_index<PERM>(p, m, n + j)] = Tr::from_float(Epi::apply(v[j], bj, d0j, d1j));
               }
             }
           }

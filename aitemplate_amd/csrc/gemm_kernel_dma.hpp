@@ -131,7 +131,7 @@ AITAMD_DEVICE void sched_step() {
   sched_spread_vmem<VM, REST, PER>();
 }
 
-template <class T, class Tile, class Epi>
+template <class T, class Tile, class Epi, bool PERM = false>
 __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const GemmParams p) {
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
@@ -323,7 +323,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;
     const T* bias = reinterpret_cast<const T*>(p.bias);
 
-    bool vec_ok = ((p.N & 7) == 0) && ((p.ldc & 7) == 0) && ((p.sc & 7) == 0) &&
+    bool vec_ok = ((p.N & 7) == 0) && ((p.ldc & 7) == 0) && ((p.sc & 7) == 0) && (!PERM || (p.perm_n2 & 7) == 0) &&
         ((reinterpret_cast<uintptr_t>(p.c) & 15) == 0);
     if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
     if (Epi::kNumD >= 1)
@@ -366,7 +366,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
           const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + row * PITCH + rd_col);
           const f32x4 v1 = *reinterpret_cast<const f32x4*>(strip + row * PITCH + rd_col + 4);
           float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-          const int64_t c_idx = (int64_t)m * p.ldc + n;
+          const int64_t c_idx = out_index<PERM>(p, m, n);
           const int64_t d_idx = (int64_t)m * p.ldd + n;
           if (vec_ok) {
             vec8 bv = {}, d0v = {}, d1v = {};
@@ -387,7 +387,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
                 if constexpr (Epi::kHasBias) bj = Tr::to_float(bias[n + j]);
                 if constexpr (Epi::kNumD >= 1) d0j = Tr::to_float(D0b[d_idx + j]);
                 if constexpr (Epi::kNumD >= 2) d1j = Tr::to_float(D1b[d_idx + j]);
-                Cb[c_idx + j] = Tr::from_float(Epi::apply(v[j], bj, d0j, d1j));
+                Cb[out_index<PERM>(p, m, n + j)] = Tr::from_float(Epi::apply(v[j], bj, d0j, d1j));
               }
             }
           }

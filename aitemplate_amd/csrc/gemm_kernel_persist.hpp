@@ -58,7 +58,7 @@ struct GemmTilePersist {
   static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
 };
 
-template <class T, class Tile, class Epi>
+template <class T, class Tile, class Epi, bool PERM = false>
 __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const GemmParams p) {
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
@@ -210,7 +210,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   // ---- epilogue -------------------------------------------------------------------------------
   const T* bias = reinterpret_cast<const T*>(p.bias);
-  bool vec_ok = ((p.N & 7) == 0) && ((p.ldc & 7) == 0) && ((p.sc & 7) == 0) &&
+  bool vec_ok = ((p.N & 7) == 0) && ((p.ldc & 7) == 0) && ((p.sc & 7) == 0) && (!PERM || (p.perm_n2 & 7) == 0) &&
       ((reinterpret_cast<uintptr_t>(p.c) & 15) == 0);
   if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
   if (Epi::kNumD >= 1)
@@ -253,7 +253,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
             *reinterpret_cast<const vec8*>(strip + row * Tile::STRIP_PITCH + ((r_c ^ (row & (SC - 1))) << 4));
         const int m = c.m0 + wm * Tile::WTM + mi * MT + row;
         if (m < p.M && n < p.N) {
-          const int64_t c_idx = (int64_t)m * p.ldc + n;
+          const int64_t c_idx = out_index<PERM>(p, m, n);
           const int64_t d_idx = (int64_t)m * p.ldd + n;
           if (vec_ok) {
             vec8 d0v = {}, d1v = {};
@@ -273,7 +273,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
                 if constexpr (Epi::kHasBias) bj = Tr::to_float(bias[n + j]);
                 if constexpr (Epi::kNumD >= 1) d0j = Tr::to_float(D0b[d_idx + j]);
                 if constexpr (Epi::kNumD >= 2) d1j = Tr::to_float(D1b[d_idx + j]);
-                Cb[c_idx + j] = Tr::from_float(Epi::apply(Tr::to_float(raw[j]), bj, d0j, d1j));
+                Cb[out_index<PERM>(p, m, n + j)] = Tr::from_float(Epi::apply(Tr::to_float(raw[j]), bj, d0j, d1j));
               }
             }
           }

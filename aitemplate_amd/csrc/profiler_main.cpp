@@ -136,7 +136,33 @@ struct OperandSet {
   DeviceBuf a, b, bias, d0, d1, c;
 };
 
-int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, int64_t N, int64_t K, bool batched) {
+// layout 0 = plain store; otherwise the permuting launcher with the op's (g1, g2, g3)
+struct PermuteSpec {
+  int layout = 0;
+  int64_t g[3] = {1, 1, 1};
+};
+
+// permuting op name -> base op (which names the epilogue) and layout id; false when `op` does not permute
+bool permute_op(const std::string& op, std::string* base, int* layout) {
+  static const struct {
+    const char* op;
+    const char* base;
+    int layout;
+  } table[] = {{"gemm_rcr_permute_m2n3", "gemm_rcr", AITAMD_PERMUTE_M2N3},
+               {"gemm_rcr_bias_permute_m2n3", "gemm_rcr_bias", AITAMD_PERMUTE_M2N3},
+               {"gemm_rcr_bias_permute_m3n2", "gemm_rcr_bias", AITAMD_PERMUTE_M3N2},
+               {"gemm_rcr_bias_permute", "gemm_rcr_bias", AITAMD_PERMUTE_M3N2}};
+  for (const auto& t : table)
+    if (op == t.op) {
+      *base = t.base;
+      *layout = t.layout;
+      return true;
+    }
+  return false;
+}
+
+int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, int64_t N, int64_t K, bool batched,
+                      const PermuteSpec& perm = PermuteSpec()) {
   const int epi = epilogue_of(op);
   if (epi < 0) {
     fprintf(stderr, "unknown op %s\n", op.c_str());
@@ -183,6 +209,9 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
   HIP_OK(hipEventCreate(&e1));
 
   auto launch = [&](int algo, const OperandSet& o) -> int {
+    if (perm.layout)
+      return aitamd_gemm_rcr_permute(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.c.p, M, N, K, K, K, perm.layout,
+                                     perm.g[0], perm.g[1], perm.g[2], stream);
     if (batched)
       return aitamd_bmm_rcr(dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, K, K, N, M * K, N * K, M * N, stream);
     return aitamd_gemm_rcr(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.d0.p, o.d1.p, o.c.p, M, N, K, K, K, N, N,
@@ -270,7 +299,7 @@ int profile_attention(int dtype, int64_t B, int64_t M, int64_t N, int64_t K, int
 
 int main(int argc, char** argv) {
   if (argc < 4) {
-    fprintf(stderr, "usage: %s gemm|bmm|attn <op> <dtype> dims...\n", argv[0]);
+    fprintf(stderr, "usage: %s gemm|gemm_permute|bmm|attn <op> <dtype> dims...\n", argv[0]);
     return 2;
   }
   const std::string kind = argv[1];
@@ -281,6 +310,19 @@ int main(int argc, char** argv) {
   if (kind == "gemm") {
     if (d.size() < 3) return 2;
     return profile_gemm_like(op, dtype, 1, d[0], d[1], d[2], false);
+  }
+  if (kind == "gemm_permute") {  // M N K g1 g2 g3
+    if (d.size() < 6) return 2;
+    std::string base;
+    PermuteSpec perm;
+    if (!permute_op(op, &base, &perm.layout)) {
+      fprintf(stderr, "%s is not a permuting op\n", op.c_str());
+      return 2;
+    }
+    perm.g[0] = d[3];
+    perm.g[1] = d[4];
+    perm.g[2] = d[5];
+    return profile_gemm_like(base, dtype, 1, d[0], d[1], d[2], false, perm);
   }
   if (kind == "bmm") {
     if (d.size() < 4) return 2;

@@ -89,6 +89,46 @@ def gemm(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor]
     return out
 
 
+def gemm_permute(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor], shape,
+                 out: Optional[torch.Tensor] = None, algo: int = -1) -> torch.Tensor:
+    """Run a permuting op (`_kernels.PERMUTE_OPS`): linear(a, b, bias) written through the op's 5-D permutation.
+
+    `shape` = (t1, t2, t3) as in the reference ops (gemm_rcr_bias_permute.py:28-76, gemm_rcr_permute.py:33-70).
+    Returns [t2, M/t1, t3, t1, N/(t2*t3)] for the m2n3 ops and [t2, M/(t1*t2), t3, t1, N/t3] for the others.
+    """
+    lib = _kernels.load()
+    epi, layout = _kernels.PERMUTE_OPS[op]
+    dtype = a.dtype
+    if dtype not in _TORCH_DTYPE_ID:
+        raise ValueError(f"unsupported dtype {dtype}")
+    for t, n in ((a, "a"), (b, "b"), (bias, "bias"), (out, "out")):
+        _check(t, n, dtype)
+    K = a.shape[-1]
+    a2 = a.reshape(-1, K)
+    M, N = a2.shape[0], b.shape[0]
+    if b.dim() != 2 or b.shape[1] != K:
+        raise ValueError(f"b must be [N, K={K}], got {tuple(b.shape)}")
+    if epi != 0 and (bias is None or bias.numel() != N):
+        raise ValueError("bias must be 1-D of size N")
+    t1, t2, t3 = (int(t) for t in shape)
+    if layout == _kernels.PERMUTE_M2N3:
+        if M % t1 or N % (t2 * t3):
+            raise ValueError(f"[{M}, {N}] does not split by shape {tuple(shape)}")
+        out_shape = (t2, M // t1, t3, t1, N // (t2 * t3))
+    else:
+        if M % (t1 * t2) or N % t3:
+            raise ValueError(f"[{M}, {N}] does not split by shape {tuple(shape)}")
+        out_shape = (t2, M // (t1 * t2), t3, t1, N // t3)
+    if out is None:
+        out = torch.empty(out_shape, dtype=dtype, device=a.device)
+    elif not out.is_contiguous() or out.numel() != M * N:
+        raise ValueError("out must be contiguous with M*N elements")
+    rc = lib.aitamd_gemm_rcr_permute(epi, _TORCH_DTYPE_ID[dtype], algo, _p(a2), _p(b), _p(bias), _p(out), M, N, K,
+                                     _row_pitch(a2, "a"), _row_pitch(b, "b"), layout, t1, t2, t3, _stream_ptr())
+    _kernels.check(rc, op)
+    return out
+
+
 def bmm_rcr(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None, algo: int = -1) -> torch.Tensor:
     """out[b] = a[b] @ b[b].T with batch broadcast when one operand is 2-D or has batch 1
     (python/aitemplate/compiler/ops/gemm_universal/bmm.py:72-90)."""

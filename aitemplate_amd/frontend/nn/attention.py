@@ -1,0 +1,76 @@
+"""nn.MultiheadAttention: packed QKV projection, fused attention, output projection.
+
+Counterpart of the ROCm branch of python/aitemplate/frontend/nn/attention.py:95-290:
+
+    qkv  = Linear(dim, 3*dim, specialization="permute", shape=(seq_len, 3, heads), layout="m2n3")
+           [B, S, dim] -> [3, B, heads, S, head_dim]        (gemm_rcr[_bias]_permute_m2n3)
+    q, k, v = split(qkv, 1, dim=0), each viewed as [B*heads, S, head_dim]
+    attn = bmm_softmax_bmm_permute(shape=(heads,), scale=head_dim**-0.5, causal)(q, k, v)
+           -> [B, S, heads, head_dim]
+    out  = Linear(dim, dim, specialization="add" if has_residual else None)(attn.reshape(B*S, dim)[, residual])
+           -> [B, S, dim]
+
+Three kernels per block: two GEMMs and one attention launch; the split and every reshape are views.
+The CUDA-only pieces of the reference module (flash attention on a packed tensor, cu_length, the
+memory-efficient kernel) have no counterpart here; `mask_seq` needs dynamic_slice / concatenate, which
+this backend does not have."""
+from ...compiler import ops
+from .dropout import Dropout
+from .linear import Linear
+from .module import Module
+
+
+class MultiheadAttention(Module):
+    r"""Multi-Head Attention: MultiHead(Q, K, V) = Concat(head_1, ..., head_h) W^O.
+
+    Args mirror the reference: dim, batch_size, seq_len, num_heads=8, qkv_bias=False, attn_drop=0.0,
+    proj_drop=0.0, has_residual=True, causal=False, mask_seq=0, use_mem_eff=False, dtype="float16".
+    Dropout probabilities are accepted and ignored (inference)."""
+
+    def __init__(self, dim, batch_size, seq_len, num_heads=8, qkv_bias=False, attn_drop=0.0, proj_drop=0.0,
+                 has_residual=True, causal=False, mask_seq=0, use_mem_eff=False, dtype="float16"):
+        super().__init__()
+        assert dim % num_heads == 0, f"dim {dim} should be divisible by num_heads {num_heads}"
+        if mask_seq:
+            raise NotImplementedError("mask_seq needs dynamic_slice and concatenate, which this backend lacks")
+        if use_mem_eff:
+            raise NotImplementedError("mem_eff_attention is a CUDA kernel of the reference; ROCm uses "
+                                      "bmm_softmax_bmm_permute")
+        self.num_heads = num_heads
+        self.scale = (dim // num_heads) ** -0.5
+        self.causal = causal
+        self.has_residual = has_residual
+        self.qkv = Linear(dim, dim * 3, bias=qkv_bias, specialization="permute", shape=(seq_len, 3, num_heads),
+                          layout="m2n3", dtype=dtype)
+        self.attn_drop = Dropout(attn_drop, dtype=dtype)
+        self.proj = Linear(dim, dim, specialization="add" if has_residual else None, dtype=dtype)
+        self.proj_drop = Dropout(proj_drop, dtype=dtype)
+
+    @staticmethod
+    def get_shape(x):
+        return [it.value() for it in x._attrs["shape"]]
+
+    def qkv_proj(self, x):
+        return self.qkv(x)
+
+    def attention(self, x):
+        """x: [3, B, heads, S, head_dim] -> [B, S, heads, head_dim]"""
+        q, k, v = ops.split()(x, 1, dim=0)
+        _, _, _, seqlen, d = self.get_shape(q)
+        op = ops.bmm_softmax_bmm_permute(shape=(self.num_heads,), scale=self.scale, causal=self.causal)
+        return op(ops.reshape()(q, [-1, seqlen, d]), ops.reshape()(k, [-1, seqlen, d]),
+                  ops.reshape()(v, [-1, seqlen, d]))
+
+    def forward(self, *args):
+        assert len(args) >= 1
+        x = args[0]
+        batch, seq, hidden = self.get_shape(x)
+        attn_output = self.attention(self.qkv_proj(x))
+        attn_output = ops.reshape()(attn_output, [batch * seq, -1])
+        if self.has_residual:
+            assert len(args) == 2
+            x = self.proj(attn_output, args[1])
+        else:
+            x = self.proj(attn_output)
+        x = self.proj_drop(x)
+        return ops.reshape()(x, [batch, seq, hidden])

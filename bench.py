@@ -198,7 +198,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--algo", type=int, default=-1, help="kernel instance index (-1: see --select)")
+    ap.add_argument("--algo", default="-1",
+                    help="kernel instance, by index or by name (default: see --select)")
     ap.add_argument("--select", choices=("profile", "heuristic"), default="profile",
                     help="how the kernel instance is chosen when --algo is not given: an untimed profiling "
                          "pass over all instances (what compile_model does) or the library's heuristic")
@@ -223,7 +224,13 @@ def main():
     _kernels.load()
 
     op, M, N, K, _ = SHAPES["c2a"]
-    algo = args.algo
+    if args.algo.lstrip("-").isdigit():
+        algo = int(args.algo)
+    else:
+        algo = _kernels.load().aitamd_gemm_find_algo(3, 0, args.algo.encode())
+        if algo < 0:
+            sys.exit(f"bench.py: no kernel instance named {args.algo}")
+    algo_given = algo >= 0
     if algo < 0 and args.select == "profile":
         algo = pick_instance(torch, eager, _kernels, "c2a")
     if algo < 0:
@@ -251,7 +258,7 @@ def main():
         "config": {"workload": "configs[1]: gemm_rcr_bias_gelu fp16 X[24576,768] W[3072,768] bias[3072], "
                                "fp32 accumulate, tanh-GELU fused, inputs resident in HBM, rotating operand sets",
                    "instance": instance, "instance_index": algo,
-                   "instance_selected_by": "--algo" if args.algo >= 0 else args.select},
+                   "instance_selected_by": "--algo" if algo_given else args.select},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(instance)},
     }

@@ -110,6 +110,23 @@ AITAMD_API int aitamd_gemm_rcr(int epilogue, int dtype, int algo,
                                int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
                                void* stream);
 
+/* gemm_rcr[_bias...] whose [M, N] result is written through one of the reference's 5-D output permutations
+ * into a contiguous buffer.  Epilogues AITAMD_EPI_NONE and AITAMD_EPI_BIAS only (the ones the permuting ops use);
+ * g = (g1, g2, g3) is the op's `shape` attribute.
+ *   AITAMD_PERMUTE_M2N3: result viewed as [M/g1, g1, g2, g3, N/(g2*g3)], written as dims (2, 0, 3, 1, 4), i.e.
+ *     [g2, M/g1, g3, g1, N/(g2*g3)].  For a packed QKV projection with g = (seq_len, 3, heads) that is
+ *     [3, batch, heads, seq_len, head_dim].
+ *   AITAMD_PERMUTE_M3N2: result viewed as [M/(g1*g2), g1, g2, g3, N/g3], written as dims (2, 0, 3, 1, 4), i.e.
+ *     [g2, M/(g1*g2), g3, g1, N/g3] (what the ROCm backend does for layout "20314" as well).
+ * Replaces the GemmPermuteM2N3 / GemmPermute instances behind gemm_rcr_bias_permute_m2n3, gemm_rcr_permute_m2n3,
+ * gemm_rcr_bias_permute_m3n2 and gemm_rcr_bias_permute
+ * (python/aitemplate/backend/rocm/gemm/gemm_rcr_bias_permute_m2n3.py:59-75, permute_common.py:20-130). */
+enum { AITAMD_PERMUTE_M2N3 = 1, AITAMD_PERMUTE_M3N2 = 2 };
+AITAMD_API int aitamd_gemm_rcr_permute(int epilogue, int dtype, int algo,
+                                       const void* a, const void* b, const void* bias, void* c,
+                                       int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                       int layout, int64_t g1, int64_t g2, int64_t g3, void* stream);
+
 /* C[b,m,n] = sum_k A[b,m,k] * B[b,n,k]; a batch stride of 0 broadcasts that
  * operand over the batch (python/aitemplate/compiler/ops/gemm_universal/bmm.py:72-90).
  * Replaces the generated bmm_rcr op function's CK call

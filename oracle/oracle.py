@@ -11,8 +11,9 @@ Two independent restatements are kept side by side:
   ``relu`` (test_gemm_bias_relu.py:64-65), GELU (test_gemm_rcr_bias_fast_gelu.py:96;
   the kernel implements the tanh form, see backend/cuda/elementwise/custom_math.cuh:828-851),
   ``linear + D0 (+ D1)`` (test_gemm_bias_broadcast.py:213-216,372-376),
-  ``bmm(Q, K^T)`` (test_bmm.py:50-51) and
-  ``softmax(Q K^T * scale) V`` with the 0213 permute (test_bmm_softmax_bmm.py:90,111-114).
+  ``bmm(Q, K^T)`` (test_bmm.py:50-51),
+  ``softmax(Q K^T * scale) V`` with the 0213 permute (test_bmm_softmax_bmm.py:90,111-114), and the
+  5-D output permutations of the permuting GEMMs (test_gemm_bias_permute.py:73-75,138-140).
 * ``c_*`` — the plain-C triple loops of ``oracle/gemm_oracle.c`` (fp32 accumulate,
   optional reference rounding points), loaded through ctypes.
 
@@ -120,6 +121,54 @@ def torch_gemm(op: str, x, w, bias=None, d0=None, d1=None) -> torch.Tensor:
     """fp32 result of reference op `op`; cast to the input dtype by the caller."""
     y = torch.nn.functional.linear(_f(x), _f(w), _f(bias) if op != "gemm_rcr" else None)
     return torch_epilogue(op, y, _f(d0), _f(d1))
+
+
+PERMUTE_OPS = {  # op -> (op that names the epilogue, layout)
+    "gemm_rcr_permute_m2n3": ("gemm_rcr", "m2n3"),
+    "gemm_rcr_bias_permute_m2n3": ("gemm_rcr_bias", "m2n3"),
+    "gemm_rcr_bias_permute_m3n2": ("gemm_rcr_bias", "m3n2"),
+    "gemm_rcr_bias_permute": ("gemm_rcr_bias", "m3n2"),  # layout "20314" on ROCm
+}
+
+
+def permute_5d(y: torch.Tensor, layout: str, shape) -> torch.Tensor:
+    """The 5-D output permutation of the permuting GEMMs applied to a [M, N] result, as the reference's
+    tests state it: m2n3 = reshape(M0, M1, N0, N1, N2).permute(2, 0, 3, 1, 4) with shape = (M1, N0, N1)
+    (tests/unittest/ops/test_gemm_bias_permute.py:34-42,73-75); m3n2 = reshape(M0, M1, M2, N0, N1)
+    .permute(2, 0, 3, 1, 4) with shape = (M1, M2, N0) (:100-108,138-140).  Returns a contiguous tensor."""
+    M, N = y.shape
+    t1, t2, t3 = (int(t) for t in shape)
+    if layout == "m2n3":
+        r = y.reshape(M // t1, t1, t2, t3, N // (t2 * t3))
+    elif layout == "m3n2":
+        r = y.reshape(M // (t1 * t2), t1, t2, t3, N // t3)
+    else:
+        raise KeyError(layout)
+    return r.permute(2, 0, 3, 1, 4).contiguous()
+
+
+def torch_gemm_permute(op: str, x, w, bias, shape) -> torch.Tensor:
+    base, layout = PERMUTE_OPS[op]
+    return permute_5d(torch_gemm(base, x.reshape(-1, x.shape[-1]), w, bias), layout, shape)
+
+
+def torch_multihead_attention(x, qkv_w, qkv_b, proj_w, proj_b, residual, num_heads: int,
+                              causal: bool = False) -> torch.Tensor:
+    """fp32 self-attention block as the reference's module test states it
+    (tests/unittest/ops/test_attention.py / frontend/nn/attention.py:150-290): packed QKV projection,
+    softmax(q k^T / sqrt(d)) v per head, output projection (+ residual).  x: [B, S, D]."""
+    B, S, D = x.shape
+    d = D // num_heads
+    qkv = torch.nn.functional.linear(_f(x), _f(qkv_w), _f(qkv_b))
+    q, k, v = qkv.reshape(B, S, 3, num_heads, d).permute(2, 0, 3, 1, 4)
+    s = torch.matmul(q, k.transpose(-1, -2)) * (d ** -0.5)
+    if causal:
+        s = s.masked_fill(torch.triu(torch.ones(S, S, dtype=torch.bool), diagonal=1), float("-inf"))
+    o = torch.matmul(torch.softmax(s, dim=-1), v).permute(0, 2, 1, 3).reshape(B * S, D)
+    y = torch.nn.functional.linear(o, _f(proj_w), _f(proj_b))
+    if residual is not None:
+        y = y + _f(residual).reshape(B * S, D)
+    return y.reshape(B, S, D)
 
 
 def torch_bmm_rcr(q, k) -> torch.Tensor:

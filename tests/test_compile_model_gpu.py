@@ -214,3 +214,103 @@ def test_benchmark_config_through_compile_model(cfg):
     # timing through the ABI works and is positive
     mean, std, _ = module.benchmark_with_tensors([inp[k].cuda() for k in order], [y], count=5, repeat=2)
     assert mean > 0
+
+
+# ---- permuting GEMMs and nn.MultiheadAttention ------------------------------------------------
+@pytest.mark.parametrize("copy_op", [False, True])
+@pytest.mark.parametrize("op_cls,layout,M,N,K,shape", [
+    ("gemm_rcr_bias_permute", "m2n3", 4 * 256, 4 * 16 * 128, 256, (256, 4, 16)),   # test_gemm_bias_permute.py:34-42
+    ("gemm_rcr_bias_permute", "m3n2", 4 * 16 * 32, 8 * 128, 256, (16, 32, 8)),     # test_gemm_bias_permute.py:100-108
+    ("gemm_rcr_bias_permute", "20314", 4 * 16 * 32, 8 * 128, 256, (16, 32, 8)),
+    ("gemm_rcr_permute", "m2n3", 4 * 256, 4 * 16 * 128, 256, (256, 4, 16)),        # test_gemm_permute.py m2n3 case
+])
+def test_gemm_permute_ops(op_cls, layout, M, N, K, shape, copy_op):
+    print(f"case compile_model {op_cls} {layout} M={M} N={N} K={K} shape={shape} copy={copy_op}", flush=True)
+    X = Tensor(shape=[M, K], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[N, K], dtype="float16", name="input_1", is_input=True)
+    ins = [X, W]
+    has_bias = op_cls == "gemm_rcr_bias_permute"
+    if has_bias:
+        ins.append(Tensor(shape=[N], dtype="float16", name="input_2", is_input=True))
+    OP = getattr(ops, op_cls)(shape, layout=layout)
+    if copy_op:
+        OP = getattr(ops, op_cls)(**OP._get_op_attributes())
+    Y = _mark_output(OP(*ins))
+    module = compile_model(Y, detect_target(), WORKDIR, f"{op_cls}_{layout}_{next(_counter)}")
+    x, w, b = _rand((M, K), 1), _rand((N, K), 2, K ** -0.5), _rand((N,), 3)
+    want = oracle.torch_gemm_permute(OP._attrs["op"], x, w, b if has_bias else None, shape).half().float()
+    y = torch.empty(tuple(want.shape), dtype=torch.float16, device="cuda")
+    feed = {"input_0": x.cuda(), "input_1": w.cuda()}
+    if has_bias:
+        feed["input_2"] = b.cuda()
+    out = module.run_with_tensors(feed, [y])
+    assert tuple(out["output_0"].shape) == tuple(want.shape)
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()
+
+
+def test_split_pieces_as_outputs_and_inputs():
+    """split is a view: pieces of an input feed GEMMs at their byte offsets, and pieces of a produced
+    tensor that are graph outputs are copied out of the producer's buffer."""
+    print("case compile_model split", flush=True)
+    P, M, K, N = 3, 64, 32, 48
+    X = Tensor(shape=[P, M, K], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[N, K], dtype="float16", name="input_1", is_input=True)
+    pieces = ops.split()(X, 1, dim=0)
+    y1 = _mark_output(ops.gemm_rcr()(ops.reshape()(pieces[2], [M, K]), W), "output_0")
+    packed = ops.gemm_rcr()(ops.reshape()(X, [P * M, K]), W)         # [P*M, N], internal
+    a, b = ops.split()(packed, [M, 2 * M], dim=0)
+    _mark_output(a, "output_1")
+    _mark_output(b, "output_2")
+    module = compile_model([y1, a, b], detect_target(), WORKDIR, f"split_{next(_counter)}")
+    x, w = _rand((P, M, K), 1), _rand((N, K), 2, K ** -0.5)
+    full = oracle.torch_gemm("gemm_rcr", x.reshape(P * M, K), w).half().float()
+    outs = [torch.empty(M, N, dtype=torch.float16, device="cuda"),
+            torch.empty(M, N, dtype=torch.float16, device="cuda"),
+            torch.empty(2 * M, N, dtype=torch.float16, device="cuda")]
+    module.run_with_tensors({"input_0": x.cuda(), "input_1": w.cuda()}, outs)
+    torch.testing.assert_close(outs[0].cpu().float(), full[2 * M:], atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(outs[1].cpu().float(), full[:M], atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(outs[2].cpu().float(), full[M:], atol=1e-2, rtol=1e-2)
+    module.close()
+
+
+@pytest.mark.parametrize("B,S,D,H,qkv_bias,residual,causal", [
+    (2, 384, 768, 12, True, True, False),      # BERT-base block shape
+    (4, 197, 768, 12, True, True, False),      # ViT-B/16 block shape: sequence tail
+    (1, 64, 512, 8, False, False, True),
+    (3, 50, 96, 4, False, True, True),
+])
+def test_nn_multihead_attention(B, S, D, H, qkv_bias, residual, causal):
+    """frontend.nn.MultiheadAttention (packed QKV GEMM with the m2n3 store, fused attention, projection with
+    the residual add) against the fp32 PyTorch block.  Tolerance 2e-2: three chained fp16 kernels, one of
+    them the softmax path."""
+    from aitemplate_amd.frontend import nn
+
+    print(f"case compile_model MultiheadAttention B={B} S={S} D={D} H={H} bias={qkv_bias} res={residual} "
+          f"causal={causal}", flush=True)
+    mha = nn.MultiheadAttention(D, B, S, H, qkv_bias=qkv_bias, has_residual=residual, causal=causal)
+    mha.name_parameter_tensor()
+    X = Tensor(shape=[B, S, D], dtype="float16", name="input_0", is_input=True)
+    args = [X]
+    if residual:
+        args.append(Tensor(shape=[B * S, D], dtype="float16", name="input_1", is_input=True))
+    Y = _mark_output(mha(*args))
+    module = compile_model(Y, detect_target(), WORKDIR, f"mha_{next(_counter)}")
+    x, res = _rand((B, S, D), 1), _rand((B * S, D), 2)
+    qkv_w, qkv_b = _rand((3 * D, D), 3, D ** -0.5), _rand((3 * D,), 4, 0.5)
+    proj_w, proj_b = _rand((D, D), 5, D ** -0.5), _rand((D,), 6, 0.5)
+    consts = {"qkv_weight": qkv_w.cuda(), "proj_weight": proj_w.cuda(), "proj_bias": proj_b.cuda()}
+    if qkv_bias:
+        consts["qkv_bias"] = qkv_b.cuda()
+    assert sorted(module.get_constant_names()) == sorted(consts)
+    module.set_many_constants_with_tensors(consts)
+    want = oracle.torch_multihead_attention(x, qkv_w, qkv_b if qkv_bias else None, proj_w, proj_b,
+                                            res if residual else None, H, causal)
+    feed = {"input_0": x.cuda()}
+    if residual:
+        feed["input_1"] = res.cuda()
+    y = torch.empty(B, S, D, dtype=torch.float16, device="cuda")
+    module.run_with_tensors(feed, [y])
+    torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
+    module.close()

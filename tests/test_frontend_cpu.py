@@ -415,3 +415,107 @@ def test_profile_results_are_cached_and_reused(tmp_path, monkeypatch):
     monkeypatch.setenv("CI_FLAG", "CIRCLECI")
     with detect_target() as target:
         assert target.get_profile_cache_path() is None
+
+
+# ---- permuting GEMMs, split, nn.MultiheadAttention ------------------------------------------
+def test_permuting_gemm_ops_shapes_names_and_copies():
+    """Shapes as in tests/unittest/ops/test_gemm_bias_permute.py:34-75 (m2n3), :100-140 (m3n2) and
+    test_gemm_permute.py of the reference."""
+    X = Tensor([4 * 256, 256], name="x", is_input=True)
+    W = Tensor([4 * 16 * 128, 256], name="w", is_input=True)
+    Bv = Tensor([4 * 16 * 128], name="b", is_input=True)
+    op = ops.gemm_rcr_bias_permute((256, 4, 16), layout="m2n3")
+    y = op(X, W, Bv)
+    assert op._attrs["op"] == "gemm_rcr_bias_permute_m2n3" and op._attrs["layout"] == "Permute5D_m2n3"
+    assert [d.value() for d in y.shape()] == [4, 4, 16, 256, 128]  # [N0, M0, N1, M1, N2]
+    assert [d.value() for d in op._attrs["outputs"][0].shape()] == [1024, 8192]
+    assert op._attrs["permute_shape"] == "256_4_16" and op._attrs["epilogue_alignment"] == 8
+    clone = ops.gemm_rcr_bias_permute(**op._get_op_attributes())
+    assert clone._attrs["op"] == op._attrs["op"] and clone._attrs["shape"] == (256, 4, 16)
+
+    X3 = Tensor([4 * 16 * 32, 256], name="x3", is_input=True)
+    W3 = Tensor([8 * 128, 256], name="w3", is_input=True)
+    B3 = Tensor([8 * 128], name="b3", is_input=True)
+    for layout, name in (("m3n2", "gemm_rcr_bias_permute_m3n2"), ("20314", "gemm_rcr_bias_permute")):
+        op3 = ops.gemm_rcr_bias_permute((16, 32, 8), layout=layout)
+        y3 = op3(X3, W3, B3)
+        assert op3._attrs["op"] == name
+        assert [d.value() for d in y3.shape()] == [32, 4, 8, 16, 128]  # [M2, M0, N0, M1, N1]
+
+    op2 = ops.gemm_rcr_permute((256, 4, 16), layout="m2n3")
+    y2 = op2(X, W)
+    assert op2._attrs["op"] == "gemm_rcr_permute_m2n3"
+    assert [d.value() for d in y2.shape()] == [4, 4, 16, 256, 128]
+    with pytest.raises(NotImplementedError):
+        ops.gemm_rcr_permute((2, 2), layout="0213")  # CUDA-only layout of the reference
+    with pytest.raises(NotImplementedError):
+        ops.gemm_rcr_bias_permute((1, 2, 3), layout="nope")
+    with pytest.raises(RuntimeError, match="does not split"):
+        ops.gemm_rcr_bias_permute((100, 4, 16), layout="m2n3")(X, W, Bv)
+    # a 3-D A folds its leading dims into M
+    y4 = ops.gemm_rcr_permute((64, 3, 2), layout="m2n3")(Tensor([5, 64, 32], name="x4", is_input=True),
+                                                        Tensor([96, 32], name="w4", is_input=True))
+    assert [d.value() for d in y4.shape()] == [3, 5, 2, 64, 16]
+    detect_target()
+    for name in ("gemm_rcr_permute_m2n3", "gemm_rcr_bias_permute", "gemm_rcr_bias_permute_m2n3",
+                 "gemm_rcr_bias_permute_m3n2"):
+        for hook in ("config", "filter", "gen_profiler", "select_algo", "gen_function", "func_decl", "func_call"):
+            assert registry.exists(f"rocm.{name}.{hook}")
+
+
+def test_split_is_a_view_with_byte_offsets():
+    x = Tensor([3, 2, 4, 8, 16], name="x", is_input=True)
+    q, k, v = ops.split()(x, 1, dim=0)
+    assert [d.value() for d in k.shape()] == [1, 2, 4, 8, 16]
+    piece = 2 * 4 * 8 * 16 * 2
+    assert [t._attrs["view_offset_bytes"] for t in (q, k, v)] == [0, piece, 2 * piece]
+    a, b = ops.split()(Tensor([1, 10, 4], name="z", is_input=True), [3, 7], dim=1)
+    assert [d.value() for d in b.shape()] == [1, 7, 4] and b._attrs["view_offset_bytes"] == 3 * 4 * 2
+    parts = ops.split()(Tensor([10, 4], name="u", is_input=True), 4)  # torch semantics: 4, 4, 2
+    assert [p.shape()[0].value() for p in parts] == [4, 4, 2]
+    with pytest.raises(NotImplementedError):
+        ops.split()(Tensor([2, 10], name="w", is_input=True), 5, dim=1)
+    with pytest.raises(RuntimeError, match="does not match"):
+        ops.split()(Tensor([10, 4], name="t", is_input=True), [3, 3], dim=0)
+    # offsets accumulate through views of views and reach the generated bindings
+    from aitemplate_amd.compiler.transform.mark_param_tensor import storage_offset_bytes
+
+    k2 = ops.reshape()(k, [-1, 8, 16])
+    assert storage_offset_bytes(k2) == piece
+
+
+def test_multihead_attention_block_compiles_to_three_kernels(tmp_path, monkeypatch):
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    reset_name_counters()
+    B, S, D, H = 2, 64, 128, 4
+    x = Tensor([B, S, D], name="x", is_input=True)
+    res = Tensor([B * S, D], name="res", is_input=True)  # same shape as the projection, as the reference requires
+    mha = nn.MultiheadAttention(D, B, S, H, qkv_bias=True)
+    mha.name_parameter_tensor()
+    y = mha(x, res)
+    y._attrs["is_output"] = True
+    y._attrs["name"] = "y"
+    assert [d.value() for d in y.shape()] == [B, S, D]
+    import torch
+
+    if torch.cuda.is_available():
+        compile_model(y, detect_target(), str(tmp_path), "mha").close()
+    else:
+        with pytest.raises(RuntimeError, match="AITemplateModelContainerCreate"):
+            compile_model(y, detect_target(), str(tmp_path), "mha")
+    build = tmp_path / "mha"
+    model_src = (build / "model-generated.cpp").read_text()
+    entries = re.findall(r'OpEntry\{"(\w+)"', model_src)
+    assert entries == ["gemm_rcr_bias_permute_m2n3_0", "bmm_softmax_bmm_permute_3", "gemm_rcr_bias_add_6"] or \
+        [e.rsplit("_", 1)[0] for e in entries] == ["gemm_rcr_bias_permute_m2n3", "bmm_softmax_bmm_permute",
+                                                   "gemm_rcr_bias_add"], entries
+    qkv_src = (build / f"{entries[0]}.cpp").read_text()
+    assert "const int p_dim0, const int p_dim1, const int p_dim2, hipStream_t stream)" in qkv_src
+    assert "aitamd_gemm_rcr_permute(1, 0, algo, a, b, bias_ptr, out_ptr, M, N, K, lda, ldb, 1, p_dim0, p_dim1, " \
+           "p_dim2, stream)" in qkv_src
+    assert f", {S}, 3, {H}, stream);" in model_src
+    # K and V are the second and third [B, heads, S, head_dim] pieces of the packed projection
+    piece = B * S * D * 2
+    assert f"+ ({piece});" in model_src and f"+ ({2 * piece});" in model_src
+    with pytest.raises(NotImplementedError):
+        nn.MultiheadAttention(D, B, S, H, mask_seq=4)

@@ -212,3 +212,67 @@ def test_config_generators_and_work_counts():
     assert oracle.config_flops_bytes("c5") == (42949672960, 20971520)
     small = oracle.config_inputs("c3", m_override=200)
     assert small["x"].shape == (200, 4096) and small["d1"].shape == (200, 1024)
+
+
+# ---- permuting GEMMs and the attention block ------------------------------------------------
+@pytest.mark.parametrize("layout,dims", [("m2n3", (3, 5, 2, 4, 6)), ("m3n2", (3, 4, 5, 2, 6)),
+                                         ("m2n3", (1, 7, 3, 1, 8)), ("m3n2", (2, 1, 3, 4, 1))])
+def test_permute_5d_matches_the_reference_stride_tables(layout, dims):
+    """Element by element against the destination strides the reference hands to its kernels
+    (python/aitemplate/backend/rocm/gemm/permute_common.py:84-91 for m2n3, :124-125 for m3n2): an
+    independent statement of the same permutation.  Unique values make any wrong index visible."""
+    if layout == "m2n3":
+        M0, M1, N0, N1, N2 = dims
+        M, N, shape = M0 * M1, N0 * N1 * N2, (M1, N0, N1)
+    else:
+        M0, M1, M2, N0, N1 = dims
+        M, N, shape = M0 * M1 * M2, N0 * N1, (M1, M2, N0)
+    y = torch.arange(M * N, dtype=torch.float32).reshape(M, N)
+    got = oracle.permute_5d(y, layout, shape).reshape(-1)
+    want = torch.full((M * N,), -1.0)
+    for m in range(M):
+        for n in range(N):
+            if layout == "m2n3":
+                m0, m1 = divmod(m, M1)
+                n0, r = divmod(n, N1 * N2)
+                n1, n2 = divmod(r, N2)
+                dst = m0 * (N1 * M1 * N2) + m1 * N2 + n0 * (M0 * N1 * M1 * N2) + n1 * (M1 * N2) + n2
+            else:
+                m0, r = divmod(m, M1 * M2)
+                m1, m2 = divmod(r, M2)
+                n0, n1 = divmod(n, N1)
+                dst = m0 * (N0 * M1 * N1) + m1 * N1 + m2 * (M0 * N0 * M1 * N1) + n0 * (M1 * N1) + n1
+            want[dst] = y[m, n]
+    assert torch.equal(got, want)
+
+
+def test_gemm_permute_for_packed_qkv_gives_per_head_projections():
+    """shape = (seq, 3, heads) on a packed projection must give [3, B, heads, S, d] with
+    out[j, b, h] = x[b] @ w[j*D + h*d : j*D + (h+1)*d].T + bias[...]: the layout the attention op reads."""
+    B, S, D, H = 2, 5, 12, 3
+    d = D // H
+    x, w, bias = _rand((B, S, D), seed=1), _rand((3 * D, D), seed=2), _rand((3 * D,), seed=3)
+    out = oracle.torch_gemm_permute("gemm_rcr_bias_permute_m2n3", x, w, bias, (S, 3, H))
+    assert tuple(out.shape) == (3, B, H, S, d)
+    for j in range(3):
+        for b in range(B):
+            for h in range(H):
+                rows = slice(j * D + h * d, j * D + (h + 1) * d)
+                want = x[b].float() @ w[rows].float().T + bias[rows].float()
+                assert torch.allclose(out[j, b, h], want, atol=1e-5)
+    no_bias = oracle.torch_gemm_permute("gemm_rcr_permute_m2n3", x, w, None, (S, 3, H))
+    assert torch.allclose(out - no_bias, bias.float().reshape(3, 1, H, 1, d).expand_as(out), atol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_block_matches_torch_nn_multiheadattention(causal):
+    """The block reduces to the library's nn.MultiheadAttention (packed in_proj, batch_first) plus a residual."""
+    B, S, D, H = 2, 7, 16, 4
+    mha = torch.nn.MultiheadAttention(D, H, bias=True, batch_first=True).eval()
+    x, res = _rand((B, S, D), torch.float32, seed=4), _rand((B * S, D), torch.float32, seed=5)
+    mask = torch.triu(torch.ones(S, S, dtype=torch.bool), diagonal=1) if causal else None
+    with torch.no_grad():
+        want, _ = mha(x, x, x, attn_mask=mask, need_weights=False)
+        got = oracle.torch_multihead_attention(x, mha.in_proj_weight, mha.in_proj_bias, mha.out_proj.weight,
+                                               mha.out_proj.bias, res, H, causal)
+    assert torch.allclose(got, want + res.reshape(B, S, D), atol=1e-5)
