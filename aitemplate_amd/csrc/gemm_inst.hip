@@ -2,6 +2,7 @@
 // Makefile with -DAITAMD_EPI=<EpilogueId> -DAITAMD_DT=<0 fp16 | 1 bf16>.
 // It instantiates every tile of gemm_tiles.inc for that pair and exports the
 // resulting launcher table under a C symbol the dispatcher looks up.
+#include <cstdlib>
 #include <mutex>
 
 #include "gemm_host.hpp"
@@ -83,6 +84,13 @@ hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
   if (attr_err != hipSuccess) return attr_err;
 
   GemmParams p = p_in;
+  // streaming stores for outputs that will not be cached anyway (the 8 L2s hold 32 MiB together); the
+  // buffer form needs one batch of the output to span less than 2 GiB
+  {
+    static const long long nt_min = getenv("AITAMD_NT_MIN_BYTES") ? atoll(getenv("AITAMD_NT_MIN_BYTES")) : (32ll << 20);
+    const long long span = p.perm_on ? (long long)p.M * p.N * 2 : ((long long)(p.M - 1) * p.ldc + p.N) * 2;
+    p.nt_store = (long long)p.M * p.N * p.batch * 2 >= nt_min && span < 0x7fffffffll;
+  }
   p.tiles_m = (p.M + Tile::BM - 1) / Tile::BM;
   p.tiles_n = (p.N + Tile::BN - 1) / Tile::BN;
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;

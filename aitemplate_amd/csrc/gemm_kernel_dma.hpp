@@ -319,6 +319,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
 
     // ---------------- epilogue: acc -> LDS (fp32, per-wave strip) -> 16-byte stores --------
     T* Cb = reinterpret_cast<T*>(p.c) + (int64_t)batch * p.sc;
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cb, kStoreRecords);
     const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)batch * p.sd : nullptr;
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;
     const T* bias = reinterpret_cast<const T*>(p.bias);
@@ -378,7 +379,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
             for (int j = 0; j < 8; ++j)
               o[j] = Tr::from_float(
                   Epi::apply(v[j], Tr::to_float(bv[j]), Tr::to_float(d0v[j]), Tr::to_float(d1v[j])));
-            *reinterpret_cast<vec8*>(Cb + c_idx) = o;
+            store_out(Cb, c_idx, o, p.nt_store != 0, rc);
           } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {

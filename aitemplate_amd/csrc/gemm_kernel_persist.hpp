@@ -224,6 +224,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   auto epilogue = [&](const TileCoord& c) {
     T* Cb = reinterpret_cast<T*>(p.c) + (int64_t)c.batch * p.sc;
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cb, kStoreRecords);
     const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)c.batch * p.sd : nullptr;
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)c.batch * p.sd : nullptr;
     const int n = c.n0 + wn * Tile::WTN + r_c * 8;  // the lane's 8 columns: the same in every pass
@@ -264,7 +265,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
             for (int j = 0; j < 8; ++j)
               o[j] = Tr::from_float(Epi::apply(Tr::to_float(raw[j]), Tr::to_float(bv[j]), Tr::to_float(d0v[j]),
                                                Tr::to_float(d1v[j])));
-            *reinterpret_cast<vec8*>(Cb + c_idx) = o;
+            store_out(Cb, c_idx, o, p.nt_store != 0, rc);
           } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
