@@ -27,10 +27,10 @@ PEAK_HBM_GBS = 8000.0
 # this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter read for the
 # 256 MiB copy of --copy-probe in the same run.  Instances never measured report null.
 MEASURED_TRAFFIC_BYTES = {
-    # FETCH_SIZE 95421.4 KiB x 2.000 (copy: 131084.6 read for 262144 KiB) + WRITE_SIZE 147456 KiB x 1.000
-    "gemm_rcr_f16_256x256x32_w2x4_dma4_o1_p1_m32_c0": 346_412_000,
-    # FETCH_SIZE 97796.0 KiB x 2.000 + WRITE_SIZE 147456 KiB x 1.000
-    "gemm_rcr_f16_256x256x32_w2x4_persist4": 351_281_000,
+    # scale factors from a 256 MiB device copy in the same run: it reads 131084.7 KiB by FETCH_SIZE (x 2.000)
+    # and writes 262144 KiB by WRITE_SIZE (x 1.000)
+    # FETCH_SIZE 88089.3 KiB x 2.000 + WRITE_SIZE 147456.3 KiB x 1.000 (with streaming output stores)
+    "gemm_rcr_f16_256x256x32_w2x4_persist4": 331_402_000,
 }
 
 SHAPES = {
