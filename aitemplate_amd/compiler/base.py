@@ -270,6 +270,37 @@ class Tensor(Node):
     def dst_ops(self):
         return self._attrs["dst_ops"]
 
+    # arithmetic builds element-wise ops (reference: compiler/base.py:958-990)
+    def _elementwise(self, func_name: str, lhs, rhs) -> "Tensor":
+        from .ops.common.elementwise import elementwise
+        from .ops.common.epilogue import FuncEnum
+
+        return elementwise(FuncEnum[func_name])(lhs, rhs)
+
+    def __add__(self, other) -> "Tensor":
+        return self._elementwise("ADD", self, other)
+
+    def __radd__(self, other) -> "Tensor":
+        return self._elementwise("ADD", other, self)
+
+    def __sub__(self, other) -> "Tensor":
+        return self._elementwise("SUB", self, other)
+
+    def __rsub__(self, other) -> "Tensor":
+        return self._elementwise("SUB", other, self)
+
+    def __mul__(self, other) -> "Tensor":
+        return self._elementwise("MUL", self, other)
+
+    def __rmul__(self, other) -> "Tensor":
+        return self._elementwise("MUL", other, self)
+
+    def __truediv__(self, other) -> "Tensor":
+        return self._elementwise("DIV", self, other)
+
+    def __rtruediv__(self, other) -> "Tensor":
+        return self._elementwise("DIV", other, self)
+
     def is_a_const_num(self) -> bool:
         return len(self._attrs["shape"]) == 0 and self._attrs["value"] is not None
 

@@ -73,6 +73,9 @@ def compile_model(
             reset_name_counters()
             graph = transform.toposort(output_tensors)
             _bind_constants(graph, constants)
+            if do_optimize_graph:
+                graph = transform.fuse_mm_elementwise(graph, output_tensors)
+            transform.check_no_elementwise_left(graph)
             transform.name_graph(graph)
             transform.mark_param_tensor(graph, output_tensors)
             transform.profile(graph, profile_dir, profile_devs, dynamic_profiling_strategy, profile_timeout)

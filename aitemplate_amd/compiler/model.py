@@ -134,6 +134,9 @@ class Model:
         self.DLL = self._DLLWrapper(lib_path)
         self.handle = ctypes.c_void_p()
         self.allocator_handle = ctypes.c_void_p()
+        # tensors bound as constants are referenced here until replaced, so that their memory outlives
+        # the caller's variables (reference: compiler/model.py:246,874-910)
+        self.torch_constant_tensors = {}
         if num_runtimes <= 0:
             raise ValueError(f"num_runtimes must be positive, but got {num_runtimes}")
         if allocator_kind is not None:
@@ -404,22 +407,27 @@ class Model:
             self.handle, ctypes.c_void_p(stream_ptr), c_names, c_tensors, ctypes.c_size_t(len(tensors)))
 
     def set_constant_with_tensor(self, name: str, tensor) -> None:
-        """Bind a torch tensor to a constant; the model keeps using that memory (keep the tensor alive)."""
+        """Bind a torch tensor to a constant; the model keeps using that memory and holds a reference to
+        the tensor in `torch_constant_tensors` until it is replaced."""
         _check_tensors_contiguous_and_on_gpu([tensor], name="constant")
         self.set_constant(name, torch_to_ait_data(tensor))
+        self.torch_constant_tensors[name] = tensor
 
     def set_many_constants_with_tensors(self, tensors: Dict[str, Any]) -> None:
         _check_tensors_contiguous_and_on_gpu(tensors, name="constants")
         self.set_many_constants({n: torch_to_ait_data(t) for n, t in tensors.items()})
+        self.torch_constant_tensors.update(tensors)
 
     def set_double_buffer_constant_with_tensor(self, name: str, tensor, stream_ptr: Optional[int] = None) -> None:
         _check_tensors_contiguous_and_on_gpu([tensor], name="constant")
         self.set_double_buffer_constant(name, torch_to_ait_data(tensor), stream_ptr)
+        self.torch_constant_tensors[name] = tensor
 
     def set_many_double_buffer_constants_with_tensors(self, tensors: Dict[str, Any],
                                                       stream_ptr: Optional[int] = None) -> None:
         _check_tensors_contiguous_and_on_gpu(tensors, name="constants")
         self.set_many_double_buffer_constants({n: torch_to_ait_data(t) for n, t in tensors.items()}, stream_ptr)
+        self.torch_constant_tensors.update(tensors)
 
     def fold_constants(self, stream_ptr: Optional[int] = None, sync: bool = True, double_buffer: bool = False) -> None:
         fn = (self.DLL.AITemplateModelContainerFoldConstantsInDoubleBuffer if double_buffer

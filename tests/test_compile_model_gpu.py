@@ -314,3 +314,34 @@ def test_nn_multihead_attention(B, S, D, H, qkv_bias, residual, causal):
     module.run_with_tensors(feed, [y])
     torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
     module.close()
+
+
+def test_unfused_ffn_graph_is_fused_into_two_gemms():
+    """A BERT feed-forward block written with plain nn.Linear and element-wise ops
+    (gelu(x W1^T + b1) W2^T + b2 + residual) compiles to gemm_rcr_bias_gelu + gemm_rcr_bias_add
+    (reference pass: compiler/transform/fuse_mm_elementwise.py) and matches the fp32 expression."""
+    from aitemplate_amd.frontend import nn
+
+    print("case compile_model fuse_mm_elementwise FFN", flush=True)
+    M, D, H = 512, 256, 1024
+    up, down = nn.Linear(D, H), nn.Linear(H, D)
+    up.name_parameter_tensor("up")
+    down.name_parameter_tensor("down")
+    X = Tensor(shape=[M, D], dtype="float16", name="input_0", is_input=True)
+    hidden = ops.elementwise(ops.FuncEnum.GELU)(up(X))
+    Y = _mark_output(down(hidden) + X)
+    name = f"ffn_{next(_counter)}"
+    module = compile_model(Y, detect_target(), WORKDIR, name)
+    model_src = open(os.path.join(WORKDIR, name, "model-generated.cpp")).read()
+    assert "gemm_rcr_bias_gelu_" in model_src and "gemm_rcr_bias_add_" in model_src and "elementwise" not in model_src
+    x = _rand((M, D), 1)
+    w1, b1 = _rand((H, D), 2, D ** -0.5), _rand((H,), 3, 0.5)
+    w2, b2 = _rand((D, H), 4, H ** -0.5), _rand((D,), 5, 0.5)
+    module.set_many_constants_with_tensors({"up_weight": w1.cuda(), "up_bias": b1.cuda(),
+                                            "down_weight": w2.cuda(), "down_bias": b2.cuda()})
+    h = oracle.torch_gemm("gemm_rcr_bias_gelu", x, w1, b1).half()
+    want = oracle.torch_gemm("gemm_rcr_bias_add", h, w2, b2, x).half().float()
+    y = torch.empty(M, D, dtype=torch.float16, device="cuda")
+    module.run_with_tensors({"input_0": x.cuda()}, [y])
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()

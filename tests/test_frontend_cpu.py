@@ -519,3 +519,111 @@ def test_multihead_attention_block_compiles_to_three_kernels(tmp_path, monkeypat
     assert f"+ ({piece});" in model_src and f"+ ({2 * piece});" in model_src
     with pytest.raises(NotImplementedError):
         nn.MultiheadAttention(D, B, S, H, mask_seq=4)
+
+
+# ---- fuse_mm_elementwise ----------------------------------------------------------------------
+def _fuse(outputs):
+    outputs = list(outputs)
+    graph = transform.fuse_mm_elementwise(transform.toposort(outputs), outputs)
+    return graph, outputs
+
+
+def _op_names(graph):
+    return [op._attrs["op"] for op in transform.get_sorted_ops(graph)]
+
+
+@pytest.mark.parametrize("funcs,fused", [
+    (("RELU",), "gemm_rcr_bias_relu"), (("SIGMOID",), "gemm_rcr_bias_sigmoid"), (("TANH",), "gemm_rcr_bias_tanh"),
+    (("GELU",), "gemm_rcr_bias_gelu"), (("FASTGELU",), "gemm_rcr_bias_fast_gelu"),
+    (("ADD",), "gemm_rcr_bias_add"), (("ADD", "ADD"), "gemm_rcr_bias_add_add"),
+    (("ADD", "RELU"), "gemm_rcr_bias_add_relu"), (("ADD", "ADD", "RELU"), "gemm_rcr_bias_add_add_relu"),
+    (("MUL",), "gemm_rcr_bias_mul"), (("MUL", "ADD"), "gemm_rcr_bias_mul_add"), (("MUL", "TANH"), "gemm_rcr_bias_mul_tanh"),
+    (("SIGMOID", "MUL"), "gemm_rcr_bias_sigmoid_mul"), (("SIGMOID", "MUL", "TANH"), "gemm_rcr_bias_sigmoid_mul_tanh"),
+])
+def test_fuse_mm_elementwise_patterns(funcs, fused):
+    """Every row of the reference's table (fuse_mm_elementwise_patterns.py:66-190) for gemm_rcr_bias."""
+    M, N, K = 32, 48, 16
+    X, W, Bv = Tensor([M, K], name="x", is_input=True), Tensor([N, K], name="w", is_input=True), \
+        Tensor([N], name="b", is_input=True)
+    y = ops.gemm_rcr_bias()(X, W, Bv)
+    residuals = []
+    for i, f in enumerate(funcs):
+        if f in ("ADD", "MUL"):
+            d = Tensor([M, N], name=f"d{i}", is_input=True)
+            residuals.append(d)
+            y = ops.elementwise(ops.FuncEnum[f])(y, d) if i % 2 == 0 else ops.elementwise(ops.FuncEnum[f])(d, y)
+        else:
+            y = ops.elementwise(ops.FuncEnum[f])(y)
+    y._attrs["is_output"] = True
+    y._attrs["name"] = "out"
+    graph, outs = _fuse([y])
+    assert _op_names(graph) == [fused]
+    out = outs[0]
+    assert out._attrs["name"] == "out" and out._attrs["is_output"] and graph[-1] is out
+    op = list(out.src_ops())[0]
+    assert op._attrs["inputs"][:3] == [X, W, Bv] and op._attrs["inputs"][3:] == residuals
+    for t in (X, W, Bv, *residuals):
+        assert list(t.dst_ops()) == [op]  # the replaced ops no longer hang off the inputs
+    transform.check_no_elementwise_left(graph)
+
+
+def test_fuse_mm_elementwise_bias_swish_operators_and_limits():
+    M, N, K = 32, 48, 16
+    X, W, Bv = Tensor([M, K], name="x", is_input=True), Tensor([N, K], name="w", is_input=True), \
+        Tensor([N], name="b", is_input=True)
+    # gemm_rcr + bias written with the + operator, then swish = x * sigmoid(x)
+    x = ops.gemm_rcr()(X, W) + Bv
+    y = x * ops.elementwise(ops.FuncEnum.SIGMOID)(x)
+    y._attrs["is_output"] = True
+    graph, outs = _fuse([y])
+    assert _op_names(graph) == ["gemm_rcr_bias_swish"]
+    # a tensor that is also a graph output, or has two consumers, ends the chain
+    h = ops.gemm_rcr_bias()(X, W, Bv)
+    h._attrs["is_output"] = True
+    r = ops.elementwise(ops.FuncEnum.RELU)(h)
+    r._attrs["is_output"] = True
+    graph, outs = _fuse([h, r])
+    assert _op_names(graph) == ["gemm_rcr_bias", "elementwise"]
+    with pytest.raises(NotImplementedError, match="could not be fused"):
+        transform.check_no_elementwise_left(graph)
+    # a residual of another shape (row broadcast) is not an epilogue of this backend
+    h2 = ops.gemm_rcr_bias()(X, W, Bv)
+    z = h2 + Tensor([1, N], name="row", is_input=True)
+    z._attrs["is_output"] = True
+    graph, outs = _fuse([z])
+    assert _op_names(graph) == ["gemm_rcr_bias", "elementwise"]
+    # the longest row wins and the rest of the chain stays: bias -> relu fused, the following tanh is left
+    h3 = ops.elementwise(ops.FuncEnum.TANH)(ops.elementwise(ops.FuncEnum.RELU)(ops.gemm_rcr_bias()(X, W, Bv)))
+    h3._attrs["is_output"] = True
+    graph, outs = _fuse([h3])
+    assert _op_names(graph) == ["gemm_rcr_bias_relu", "elementwise"]
+    # scalars are accepted by the op and broadcasting follows numpy
+    s = ops.elementwise(ops.FuncEnum.MUL)(Tensor([4, 1, 8], name="a", is_input=True), Tensor([5, 1], name="c", is_input=True))
+    assert [d.value() for d in s.shape()] == [4, 5, 8]
+    assert (2.0 * X)._attrs["src_ops"] and list((X / 2).src_ops())[0]._attrs["func"] == ops.FuncEnum.DIV
+    with pytest.raises(RuntimeError, match="not compatible"):
+        ops.elementwise(ops.FuncEnum.ADD)(Tensor([4, 3], name="p", is_input=True), Tensor([4, 2], name="q", is_input=True))
+
+
+def test_compile_model_runs_the_fusion_pass_and_rejects_leftovers(tmp_path, monkeypatch):
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    reset_name_counters()
+    X = Tensor([64, 32], name="x", is_input=True)
+    lin = nn.Linear(32, 48)
+    lin.name_parameter_tensor("fc")
+    y = ops.elementwise(ops.FuncEnum.RELU)(lin(X))
+    y._attrs["is_output"] = True
+    y._attrs["name"] = "y"
+    import torch
+
+    if torch.cuda.is_available():
+        compile_model(y, detect_target(), str(tmp_path), "fused").close()
+    else:
+        with pytest.raises(RuntimeError, match="AITemplateModelContainerCreate"):
+            compile_model(y, detect_target(), str(tmp_path), "fused")
+    model_src = (tmp_path / "fused" / "model-generated.cpp").read_text()
+    assert re.findall(r'OpEntry\{"(\w+)"', model_src) == ["gemm_rcr_bias_relu_0"]
+    z = ops.elementwise(ops.FuncEnum.EXP)(nn.Linear(32, 48)(Tensor([64, 32], name="x2", is_input=True)))
+    z._attrs["is_output"] = True
+    with pytest.raises(NotImplementedError, match="could not be fused"):
+        compile_model(z, detect_target(), str(tmp_path), "leftover")
