@@ -59,7 +59,9 @@ std::vector<uint64_t> ModelBase::CurrentSignature() const {
   return sig;
 }
 
-void ModelBase::Run(StreamType stream, bool graph_mode) {
+void ModelBase::MarkFinished(StreamType stream) { AIT_DEVICE_CHECK(hipEventRecord(run_finished_, stream)); }
+
+void ModelBase::Run(StreamType stream, bool graph_mode, bool mark_finished) {
   SetUpInputsOutputs();
   if (!graph_mode) {
     RunImpl(stream);
@@ -91,7 +93,7 @@ void ModelBase::Run(StreamType stream, bool graph_mode) {
     AIT_DEVICE_CHECK(hipGraphLaunch(graph_exec_, stream));
   }
   DeviceToDeviceCopies(stream);
-  AIT_DEVICE_CHECK(hipEventRecord(run_finished_, stream));
+  if (mark_finished) MarkFinished(stream);
 }
 
 void ModelBase::Profile(StreamType stream, size_t iters, const std::string& filename) {

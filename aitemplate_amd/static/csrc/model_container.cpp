@@ -228,26 +228,37 @@ void ModelContainer::Profile(const AITData* inputs, size_t num_inputs, AITData* 
   ReturnModel(m, false);
 }
 
+// One runtime, prepared once, run `count` times back to back between two events - no per-run wait, as in
+// the reference (static/csrc/model_container.cpp:856-900).
 float ModelContainer::BenchmarkImpl(const AITData* inputs, size_t num_inputs, AITData* outputs, size_t num_outputs,
                                     StreamType stream, bool graph_mode, size_t count, int64_t** output_shapes_out) {
-  hipEvent_t e0, e1;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
   AIT_DEVICE_CHECK(hipEventCreate(&e0));
   AIT_DEVICE_CHECK(hipEventCreate(&e1));
   float ms = 0.f;
+  std::shared_lock<std::shared_mutex> constants_lk(constants_mutex_);
+  ModelBase* m = GetAvailableModel();
   try {
-    // one untimed run warms code and caches
-    Run(inputs, num_inputs, outputs, num_outputs, stream, true, graph_mode, nullptr);
+    PrepareForRun(m, inputs, num_inputs, outputs, num_outputs);
+    m->Run(stream, graph_mode);  // one untimed run warms code and caches
     AIT_DEVICE_CHECK(hipEventRecord(e0, stream));
-    for (size_t i = 0; i < count; ++i)
-      Run(inputs, num_inputs, outputs, num_outputs, stream, false, graph_mode, i + 1 == count ? output_shapes_out : nullptr);
+    // the timed runs are queued without a completion marker in between; the runtime is marked once
+    for (size_t i = 0; i < count; ++i) m->Run(stream, graph_mode, /*mark_finished=*/false);
     AIT_DEVICE_CHECK(hipEventRecord(e1, stream));
+    m->MarkFinished(stream);
+    if (output_shapes_out != nullptr) {
+      for (size_t i = 0; i < num_outputs; ++i)
+        if (output_shapes_out[i] != nullptr) m->GetOutputShape(i, output_shapes_out[i]);
+    }
     AIT_DEVICE_CHECK(hipEventSynchronize(e1));
     AIT_DEVICE_CHECK(hipEventElapsedTime(&ms, e0, e1));
   } catch (...) {
+    ReturnModel(m, /*failed=*/true);
     hipEventDestroy(e0);
     hipEventDestroy(e1);
     throw;
   }
+  ReturnModel(m, /*failed=*/false);
   hipEventDestroy(e0);
   hipEventDestroy(e1);
   return count ? ms / count : 0.f;

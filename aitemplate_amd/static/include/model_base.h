@@ -86,7 +86,9 @@ class ModelBase {
   ModelBase(const ModelBase&) = delete;
   ModelBase& operator=(const ModelBase&) = delete;
 
-  void Run(StreamType stream, bool graph_mode);
+  // `mark_finished` = false leaves out the completion event (callers that run a batch and mark its end once)
+  void Run(StreamType stream, bool graph_mode, bool mark_finished = true);
+  void MarkFinished(StreamType stream);
   void Profile(StreamType stream, size_t iters, const std::string& filename);
   bool IsPending();
   void WaitForCompletion();

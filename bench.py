@@ -160,10 +160,12 @@ def in_abi(torch, count=100):
     (x, w, b, _, out), = _make_pool(torch, op, M, N, K, 0, pool_bytes=0)[:1]
     with tempfile.TemporaryDirectory(prefix="aitamd_bench_") as tmp:
         with compile_model(Y, detect_target(), tmp, "bench_c2a") as module:
-            module.benchmark_with_tensors([x, w, b], [out], count=10)
-            ms, _, _ = module.benchmark_with_tensors([x, w, b], [out], count=count)
+            # the GPU has idled through the build: one untimed batch brings the clocks back up
+            module.benchmark_with_tensors([x, w, b], [out], count=count)
+            ms = sorted(module.benchmark_with_tensors([x, w, b], [out], count=count)[0] for _ in range(3))[1]
     return {"ms_per_run": round(ms, 5), "tflops": round(2 * M * N * K / (ms * 1e-3) / 1e12, 2),
-            "via": f"compile_model + AITemplateModelContainerBenchmark, count={count}, one fixed operand set"}
+            "via": f"compile_model + AITemplateModelContainerBenchmark, median of 3 batches of count={count} after "
+                   "one untimed batch, one fixed operand set"}
 
 
 def cpu_baseline(torch, max_seconds=20.0):
