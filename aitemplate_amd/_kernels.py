@@ -50,6 +50,7 @@ DTYPE_ID = {"float16": 0, "bfloat16": 1}
 # On ROCm the reference lowers layout "20314" like "m3n2" (gemm_rcr_bias_permute.py:66-72 of
 # python/aitemplate/compiler/ops/gemm_universal/).
 PERMUTE_M2N3, PERMUTE_M3N2 = 1, 2
+BMM_PERMUTE_OPS = ("bmm_rcr_permute",)  # epilogue 0, launched through aitamd_bmm_rcr_permute
 PERMUTE_OPS = {
     "gemm_rcr_permute_m2n3": (0, PERMUTE_M2N3),
     "gemm_rcr_bias_permute_m2n3": (1, PERMUTE_M2N3),
@@ -68,6 +69,7 @@ EXPORTED_SYMBOLS = [
     "aitamd_gemm_heuristic_algo",
     "aitamd_gemm_rcr",
     "aitamd_gemm_rcr_permute",
+    "aitamd_bmm_rcr_permute",
     "aitamd_bmm_rcr",
     "aitamd_bmm_softmax_bmm_permute",
 ]
@@ -111,6 +113,8 @@ def load() -> ctypes.CDLL:
         lib.aitamd_gemm_rcr.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]
         lib.aitamd_gemm_rcr_permute.restype = i32
         lib.aitamd_gemm_rcr_permute.argtypes = [i32, i32, i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, i64, i64, i64, vp]
+        lib.aitamd_bmm_rcr_permute.restype = i32
+        lib.aitamd_bmm_rcr_permute.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
         lib.aitamd_bmm_rcr.restype = i32
         lib.aitamd_bmm_rcr.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
         lib.aitamd_bmm_softmax_bmm_permute.restype = i32

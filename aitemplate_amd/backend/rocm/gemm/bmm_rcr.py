@@ -1,5 +1,6 @@
-"""Registry hooks of bmm_rcr.  Replaces python/aitemplate/backend/rocm/gemm/bmm_rcr.py:27-182 and
-bmm_common.py:22-363: same launcher signature (3-D dim pointers), batch strides derived from the
+"""Registry hooks of bmm_rcr and bmm_rcr_permute.  Replaces python/aitemplate/backend/rocm/gemm/bmm_rcr.py:27-182,
+bmm_rcr_permute.py and bmm_common.py:22-363 / bmm_permute_common.py:22-80: same launcher signature (3-D dim
+pointers; bmm_rcr_permute adds `const int p_dim0` = d1 before the stream), batch strides derived from the
 operand ranks (a 2-D or batch-1 operand broadcasts with stride 0)."""
 from typing import Any, Dict
 
@@ -11,10 +12,15 @@ def _config(func_attrs, dtype="float16"):
     common.gemm_config(func_attrs, dtype, "bmm")
 
 
-def _signature(func_name: str, ranks) -> str:
+def _signature(func_name: str, ranks, permute: bool = False) -> str:
     ptrs = ["void* in_ptr", "void* weight_ptr", "void* out_ptr"]
     dims = [f"int64_t* {n}" for prefix, r in zip("abc", ranks) for n in common.dim_param_names(prefix, r)]
-    return f"void {func_name}({', '.join(ptrs + dims + ['hipStream_t stream'])})"
+    pdims = ["const int p_dim0"] if permute else []
+    return f"void {func_name}({', '.join(ptrs + dims + pdims + ['hipStream_t stream'])})"
+
+
+def _is_permute(func_attrs) -> bool:
+    return func_attrs["op"] == "bmm_rcr_permute"
 
 
 def _ranks(func_attrs):
@@ -34,18 +40,23 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
     # an operand broadcasts when it is 2-D or its batch dim is 1 while B > 1
     a_batch = "(*a_dim0)" if ra == 3 else "1"
     b_batch = "(*b_dim0)" if rb == 3 else "1"
+    permute = _is_permute(func_attrs)
+    if permute and (off_c or ldc is not None):
+        raise NotImplementedError("bmm_rcr_permute writes a contiguous permuted buffer; its output cannot be a view")
     launches = []
     for key, item in func_attrs["exec_path"].items():
         if not item.algo:
             raise RuntimeError(f"{func_name}: workload {key} has no kernel instance; run profiling first")
+        call = (f"aitamd_bmm_rcr_permute({dtype}, algo, a, b, c, B, M, N, K, lda, ldb, stride_a, stride_b, p_dim0, stream)"
+                if permute else
+                f"aitamd_bmm_rcr({dtype}, algo, a, b, c, B, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, stream)")
         program = (
             f'static const int algo = resolve_instance(0, {dtype}, "{item.algo}");\n'
-            f"    check_rc(aitamd_bmm_rcr({dtype}, algo, a, b, c, B, M, N, K, lda, ldb, ldc, stride_a, stride_b, "
-            f'stride_c, stream), "{func_name}");'
+            f'    check_rc({call}, "{func_name}");'
         )
         launches.append(exec_cond_template.format(indent="  ", cond=item.exec_cond, program=program))
     return f"""{common.HEADER}
-{_signature(func_name, (ra, rb, rc))} {{
+{_signature(func_name, (ra, rb, rc), permute)} {{
 {shape_code}
   const uint16_t* a = static_cast<const uint16_t*>(in_ptr) + {off_a};
   const uint16_t* b = static_cast<const uint16_t*>(weight_ptr) + {off_b};
@@ -59,14 +70,14 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
   if (B == 0 || M == 0 || N == 0) return;
 {"".join(launches)}
   throw std::runtime_error(
-      "Unsupported workload for this bmm_rcr specialization: B=" + std::to_string(B) + " M=" + std::to_string(M) +
+      "Unsupported workload for this {func_attrs["op"]} specialization: B=" + std::to_string(B) + " M=" + std::to_string(M) +
       " N=" + std::to_string(N) + " K=" + std::to_string(K));
 }}
 {common.FOOTER}"""
 
 
 def func_decl(func_attrs) -> str:
-    return _signature(func_attrs["name"], _ranks(func_attrs)) + ";"
+    return _signature(func_attrs["name"], _ranks(func_attrs), _is_permute(func_attrs)) + ";"
 
 
 def func_call(func_attrs, indent="  ") -> str:
@@ -76,14 +87,20 @@ def func_call(func_attrs, indent="  ") -> str:
     for acc in (func_attrs["input_accessors"][0], func_attrs["input_accessors"][1],
                 func_attrs["output_accessors"][0]):
         dims += ["&" + d._attrs["name"] for d in acc.original_shapes]
-    args = [a._attrs["name"], b._attrs["name"], c._attrs["name"]] + dims + ["stream"]
+    pdims = [str(int(func_attrs["shape"][0]))] if _is_permute(func_attrs) else []
+    args = [a._attrs["name"], b._attrs["name"], c._attrs["name"]] + dims + pdims + ["stream"]
     return f"{indent}{func_attrs['name']}({', '.join(args)});"
 
 
-registry.reg("rocm.bmm_rcr.config", _config)
-registry.reg("rocm.bmm_rcr.filter", common.gemm_filter)
-registry.reg("rocm.bmm_rcr.gen_profiler", common.gemm_gen_profiler)
-registry.reg("rocm.bmm_rcr.select_algo", common.gemm_select_algo)
-registry.reg("rocm.bmm_rcr.gen_function", gen_function)
-registry.reg("rocm.bmm_rcr.func_decl", func_decl)
-registry.reg("rocm.bmm_rcr.func_call", func_call)
+def _config_permute(func_attrs, dtype="float16"):
+    common.gemm_config(func_attrs, dtype, "bmm_permute")
+
+
+for _op, _cfg in (("bmm_rcr", _config), ("bmm_rcr_permute", _config_permute)):
+    registry.reg(f"rocm.{_op}.config", _cfg)
+    registry.reg(f"rocm.{_op}.filter", common.gemm_filter)
+    registry.reg(f"rocm.{_op}.gen_profiler", common.gemm_gen_profiler)
+    registry.reg(f"rocm.{_op}.select_algo", common.gemm_select_algo)
+    registry.reg(f"rocm.{_op}.gen_function", gen_function)
+    registry.reg(f"rocm.{_op}.func_decl", func_decl)
+    registry.reg(f"rocm.{_op}.func_call", func_call)

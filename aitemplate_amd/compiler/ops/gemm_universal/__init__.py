@@ -1,4 +1,4 @@
-from .bmm import bmm, bmm_rcr  # noqa: F401
+from .bmm import bmm, bmm_rcr, bmm_rcr_permute  # noqa: F401
 from .bmm_softmax_bmm import bmm_softmax_bmm  # noqa: F401
 from .bmm_softmax_bmm_permute import bmm_softmax_bmm_permute  # noqa: F401
 from .gemm_common import gemm  # noqa: F401

@@ -1,10 +1,11 @@
-"""Batched GEMM: the bmm base class and bmm_rcr.
+"""Batched GEMM: the bmm base class, bmm_rcr and bmm_rcr_permute.
 
 Counterparts: python/aitemplate/compiler/ops/gemm_universal/bmm.py:69-119 (base, batch
 broadcast rules) and bmm_xxx.py:22-150,261-278 (layout bookkeeping; only the r-c-r
 layout exists on this backend)."""
-from ...base import Tensor
+from ...base import IntImm, Tensor
 from ...dtype import is_same_dtype
+from ...tensor_accessor import TensorAccessor
 from . import gemm_common as common
 
 
@@ -72,3 +73,41 @@ class bmm_rcr(bmm):
             "K": [common.DimInfo(common.Source.INPUT, tensor_idx=0, dim_idx=ra - 1),
                   common.DimInfo(common.Source.INPUT, tensor_idx=1, dim_idx=rb - 1)],
         }
+
+
+class bmm_rcr_permute(bmm_rcr):
+    """bmm_rcr whose [B, M, N] result is stored as reshape(B // d1, d1, M, N).permute(0, 2, 1, 3), i.e.
+    [B // d1, M, d1, N], with shape = (d1,) (layout "0213" only).
+    Counterpart of python/aitemplate/compiler/ops/gemm_universal/bmm_rcr_permute.py:28-116."""
+
+    def __init__(self, shape, layout="0213"):
+        super().__init__()
+        self._attrs["op"] = "bmm_rcr_permute"
+        self._attrs["shape"] = tuple(int(v) for v in shape)
+        self._attrs["layout"] = "Permute4DBMM_{}".format(layout)
+        self._attrs["permute_shape"] = "_".join(map(str, shape))
+
+    def __call__(self, a: Tensor, b: Tensor) -> Tensor:
+        from ..common.view_ops import reshape
+
+        if self._attrs["layout"] != "Permute4DBMM_0213":
+            raise NotImplementedError("{} is not implemented!".format(self._attrs["layout"]))
+        a, b = self._align_ab(a, b)
+        self._attrs["inputs"] = [a, b]
+        self._attrs["input_accessors"] = [TensorAccessor(a), TensorAccessor(b)]
+        self._set_depth()
+        self._sanity_check(a, b)
+        output_shape = self._infer_shapes(a, b)
+        output = Tensor(output_shape, src_ops={self}, dtype=a.dtype())
+        self._attrs["outputs"] = [output]
+        self._attrs["output_accessors"] = [TensorAccessor(output)]
+        batch, m, n = output_shape
+        d1 = self._attrs["shape"][0]
+        if not isinstance(batch, IntImm) or batch.value() % d1 != 0:
+            raise RuntimeError(f"bmm_rcr_permute needs a static batch that is a multiple of {d1}, got {batch}")
+        permuted = [batch.value() // d1, m, d1, n]
+        self._extract_epilogue_alignment(permuted)
+        return reshape()(output, permuted)
+
+    def _get_op_attributes(self):
+        return {"layout": self._attrs["layout"].split("_")[-1], "shape": self._attrs["shape"]}

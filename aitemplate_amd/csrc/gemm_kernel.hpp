@@ -45,7 +45,18 @@ struct GemmParams {
   // too large to be still cached when a consumer runs; such stores do not push the operand tiles out of
   // the L2 and reach HBM at a higher rate (bmm_rcr 768x384x384x64: 4.1 -> 6.4 TB/s).
   int32_t nt_store;
+  // Batched output whose batch index splits as b = b0 * batch_inner + b1 (0: plain batch stride sc): batch b
+  // starts at element b0 * sc_outer + b1 * sc.  This is the [B/d1, d1, M, N] -> [B/d1, M, d1, N] store of
+  // bmm_rcr_permute with batch_inner = d1, sc = N, sc_outer = M * d1 * N and ldc = d1 * N.
+  int32_t batch_inner;
+  int64_t sc_outer;
 };
+
+AITAMD_DEVICE int64_t out_batch_offset(const GemmParams& p, int batch) {
+  if (p.batch_inner == 0) return (int64_t)batch * p.sc;
+  const int b0 = batch / p.batch_inner;
+  return b0 * p.sc_outer + (batch - b0 * p.batch_inner) * p.sc;
+}
 
 // Output store of 8 or 16 bytes at element `idx` of the buffer `rc` describes (base `base`).  The streaming
 // form is a buffer store with the non-temporal bit; it is a different instruction from the plain store on
@@ -264,7 +275,7 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
     }
 
     // ---------------- epilogue: registers -> fp32 math -> 8-byte stores -------------
-    T* Cb = reinterpret_cast<T*>(p.c) + (int64_t)batch * p.sc;
+    T* Cb = reinterpret_cast<T*>(p.c) + out_batch_offset(p, batch);
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cb, kStoreRecords);
     const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)batch * p.sd : nullptr;
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;

@@ -318,7 +318,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     __builtin_amdgcn_s_barrier();
 
     // ---------------- epilogue: acc -> LDS (fp32, per-wave strip) -> 16-byte stores --------
-    T* Cb = reinterpret_cast<T*>(p.c) + (int64_t)batch * p.sc;
+    T* Cb = reinterpret_cast<T*>(p.c) + out_batch_offset(p, batch);
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cb, kStoreRecords);
     const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)batch * p.sd : nullptr;
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;

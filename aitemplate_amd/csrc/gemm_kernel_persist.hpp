@@ -223,7 +223,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   const int r_c = lane % SC;
 
   auto epilogue = [&](const TileCoord& c) {
-    T* Cb = reinterpret_cast<T*>(p.c) + (int64_t)c.batch * p.sc;
+    T* Cb = reinterpret_cast<T*>(p.c) + out_batch_offset(p, c.batch);
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cb, kStoreRecords);
     const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)c.batch * p.sd : nullptr;
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)c.batch * p.sd : nullptr;

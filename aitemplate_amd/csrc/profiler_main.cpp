@@ -209,9 +209,11 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
   HIP_OK(hipEventCreate(&e1));
 
   auto launch = [&](int algo, const OperandSet& o) -> int {
-    if (perm.layout)
+    if (perm.layout && !batched)
       return aitamd_gemm_rcr_permute(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.c.p, M, N, K, K, K, perm.layout,
                                      perm.g[0], perm.g[1], perm.g[2], stream);
+    if (batched && perm.layout)  // bmm_rcr_permute: perm.g[0] = d1
+      return aitamd_bmm_rcr_permute(dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, K, K, M * K, N * K, perm.g[0], stream);
     if (batched)
       return aitamd_bmm_rcr(dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, K, K, N, M * K, N * K, M * N, stream);
     return aitamd_gemm_rcr(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.d0.p, o.d1.p, o.c.p, M, N, K, K, K, N, N,
@@ -299,7 +301,7 @@ int profile_attention(int dtype, int64_t B, int64_t M, int64_t N, int64_t K, int
 
 int main(int argc, char** argv) {
   if (argc < 4) {
-    fprintf(stderr, "usage: %s gemm|gemm_permute|bmm|attn <op> <dtype> dims...\n", argv[0]);
+    fprintf(stderr, "usage: %s gemm|gemm_permute|bmm|bmm_permute|attn <op> <dtype> dims...\n", argv[0]);
     return 2;
   }
   const std::string kind = argv[1];
@@ -327,6 +329,13 @@ int main(int argc, char** argv) {
   if (kind == "bmm") {
     if (d.size() < 4) return 2;
     return profile_gemm_like(op, dtype, d[0], d[1], d[2], d[3], true);
+  }
+  if (kind == "bmm_permute") {  // B M N K d1
+    if (d.size() < 5) return 2;
+    PermuteSpec perm;
+    perm.layout = 1;
+    perm.g[0] = d[4];
+    return profile_gemm_like("bmm_rcr", dtype, d[0], d[1], d[2], d[3], true, perm);
   }
   if (kind == "attn") {
     if (d.size() < 6) return 2;

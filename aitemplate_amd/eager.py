@@ -157,6 +157,40 @@ def bmm_rcr(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None
     return out
 
 
+def bmm_rcr_permute(a: torch.Tensor, b: torch.Tensor, shape, out: Optional[torch.Tensor] = None,
+                    algo: int = -1) -> torch.Tensor:
+    """bmm_rcr stored as [B // d1, M, d1, N] with shape = (d1,)
+    (python/aitemplate/compiler/ops/gemm_universal/bmm_rcr_permute.py:28-116)."""
+    lib = _kernels.load()
+    dtype = a.dtype
+    for t, n in ((a, "a"), (b, "b"), (out, "out")):
+        _check(t, n, dtype)
+    a3 = a if a.dim() == 3 else a.unsqueeze(0)
+    b3 = b if b.dim() == 3 else b.unsqueeze(0)
+    if not (a3.is_contiguous() and b3.is_contiguous()):
+        raise ValueError("bmm_rcr_permute operands must be contiguous")
+    B = max(a3.shape[0], b3.shape[0])
+    if a3.shape[0] not in (1, B) or b3.shape[0] not in (1, B):
+        raise ValueError("batch sizes must match or be 1")
+    M, K = a3.shape[1], a3.shape[2]
+    N = b3.shape[1]
+    if b3.shape[2] != K:
+        raise ValueError("K mismatch")
+    d1 = int(shape[0])
+    if d1 <= 0 or B % d1:
+        raise ValueError(f"batch {B} is not a multiple of d1 = {d1}")
+    if out is None:
+        out = torch.empty(B // d1, M, d1, N, dtype=dtype, device=a.device)
+    elif not out.is_contiguous() or out.numel() != B * M * N:
+        raise ValueError("out must be contiguous with B*M*N elements")
+    sa = 0 if (a3.shape[0] == 1 and B > 1) else M * K
+    sb = 0 if (b3.shape[0] == 1 and B > 1) else N * K
+    rc = lib.aitamd_bmm_rcr_permute(_TORCH_DTYPE_ID[dtype], algo, _p(a3), _p(b3), _p(out), B, M, N, K, K, K, sa, sb,
+                                    d1, _stream_ptr())
+    _kernels.check(rc, "bmm_rcr_permute")
+    return out
+
+
 def bmm_softmax_bmm_permute(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, shape, scale: float = 1.0,
                             causal: bool = False, layout: str = "0213",
                             out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -138,6 +138,15 @@ AITAMD_API int aitamd_bmm_rcr(int dtype, int algo,
                               int64_t stride_a, int64_t stride_b, int64_t stride_c,
                               void* stream);
 
+/* bmm_rcr whose [B, M, N] result, viewed as [B/d1, d1, M, N], is written as [B/d1, M, d1, N] (the reference's
+ * "0213" permutation with shape = (d1,)): rows of one (batch, head) pair are d1*N elements apart.
+ * Replaces the DeviceBatchedGemmEPermuteXdl instances behind bmm_rcr_permute
+ * (python/aitemplate/backend/rocm/gemm/bmm_rcr_permute.py, bmm_permute_common.py:29-56). */
+AITAMD_API int aitamd_bmm_rcr_permute(int dtype, int algo, const void* a, const void* b, void* c,
+                                      int64_t batch, int64_t M, int64_t N, int64_t K,
+                                      int64_t lda, int64_t ldb, int64_t stride_a, int64_t stride_b,
+                                      int64_t d1, void* stream);
+
 /* out[b / G, m, b % G, o] = sum_n softmax_n( scale * sum_k Q[b,m,k] K[b,n,k] ) V[b,n,o]
  * Q [B,M,K], K [B,N,K], V [B,N,O] contiguous; out [B/G, M, G, O] (the "0213"
  * permute of [B/G, G, M, O]); G = number of heads, B % G == 0.  `scale` is

@@ -180,6 +180,14 @@ def torch_bmm_rcr(q, k) -> torch.Tensor:
     return torch.matmul(q, k.transpose(-1, -2))
 
 
+def torch_bmm_rcr_permute(q, k, d1: int) -> torch.Tensor:
+    """bmm(Q, K^T).reshape(B // d1, d1, M, N).permute(0, 2, 1, 3), as the reference's op states it
+    (python/aitemplate/compiler/ops/gemm_universal/bmm_rcr_permute.py:36-45, tests/unittest/ops/test_bmm_permute.py)."""
+    y = torch_bmm_rcr(q, k)
+    B, M, N = y.shape
+    return y.reshape(B // d1, d1, M, N).permute(0, 2, 1, 3).contiguous()
+
+
 def torch_bmm_softmax_bmm_permute(q, k, v, scale: float, num_heads: int, causal: bool = False,
                                   chunk: int = 4) -> torch.Tensor:
     """softmax(Q K^T * scale) V, output [B/G, M, G, O]; chunked over the batch to bound memory."""

@@ -345,3 +345,23 @@ def test_unfused_ffn_graph_is_fused_into_two_gemms():
     module.run_with_tensors({"input_0": x.cuda()}, [y])
     torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
     module.close()
+
+
+@pytest.mark.parametrize("B,M,N,K,d1,copy_op", [(24, 80, 64, 88, 12, False), (100, 88, 64, 88, 10, False),
+                                                (100, 88, 64, 88, 10, True), (10240, 88, 64, 88, 10, False)])
+def test_bmm_rcr_permute(B, M, N, K, d1, copy_op):      # tests/unittest/ops/test_bmm_permute.py:76-117
+    print(f"case compile_model bmm_rcr_permute B={B} M={M} N={N} K={K} d1={d1} copy={copy_op}", flush=True)
+    X = Tensor(shape=[B, M, K], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[B, N, K], dtype="float16", name="input_1", is_input=True)
+    OP = ops.bmm_rcr_permute(shape=(d1,))
+    if copy_op:
+        OP = ops.bmm_rcr_permute(**OP._get_op_attributes())
+    Y = _mark_output(OP(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"bmm_rcr_permute_{next(_counter)}")
+    q, k = _rand((B, M, K), 1), _rand((B, N, K), 2, K ** -0.5)
+    y = torch.empty(B // d1, M, d1, N, dtype=torch.float16, device="cuda")
+    out = module.run_with_tensors({"input_0": q.cuda(), "input_1": k.cuda()}, [y])
+    assert tuple(out["output_0"].shape) == (B // d1, M, d1, N)
+    want = oracle.torch_bmm_rcr_permute(q, k, d1).half().float()
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()

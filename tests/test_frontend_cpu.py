@@ -463,6 +463,24 @@ def test_permuting_gemm_ops_shapes_names_and_copies():
             assert registry.exists(f"rocm.{name}.{hook}")
 
 
+def test_bmm_rcr_permute_op_attrs():
+    op = ops.bmm_rcr_permute(shape=(12,))
+    y = op(Tensor([24, 80, 88], name="q", is_input=True), Tensor([24, 64, 88], name="k", is_input=True))
+    assert [d.value() for d in y.shape()] == [2, 80, 12, 64]
+    assert [d.value() for d in op._attrs["outputs"][0].shape()] == [24, 80, 64]
+    assert op._attrs["op"] == "bmm_rcr_permute" and op._attrs["permute_shape"] == "12"
+    assert ops.bmm_rcr_permute(**op._get_op_attributes())._attrs["shape"] == (12,)
+    with pytest.raises(NotImplementedError):
+        ops.bmm_rcr_permute(shape=(2,), layout="0321")(Tensor([4, 8, 8], name="a", is_input=True),
+                                                      Tensor([4, 8, 8], name="b", is_input=True))
+    with pytest.raises(RuntimeError, match="multiple"):
+        ops.bmm_rcr_permute(shape=(5,))(Tensor([24, 8, 8], name="a2", is_input=True),
+                                        Tensor([24, 8, 8], name="b2", is_input=True))
+    detect_target()
+    for hook in ("config", "filter", "gen_profiler", "select_algo", "gen_function", "func_decl", "func_call"):
+        assert registry.exists(f"rocm.bmm_rcr_permute.{hook}")
+
+
 def test_split_is_a_view_with_byte_offsets():
     x = Tensor([3, 2, 4, 8, 16], name="x", is_input=True)
     q, k, v = ops.split()(x, 1, dim=0)

@@ -96,3 +96,44 @@ def test_argument_errors():
                                        12, 24, 8, 8, 8, 1, 4, 3, 2, None) != 0           # bias missing
     assert lib.aitamd_gemm_rcr_permute(1, 0, -1, *args, 1, 4, 3, 2, None) == 0
     torch.cuda.synchronize()
+
+
+# ---- bmm_rcr_permute ------------------------------------------------------------------------
+@pytest.mark.parametrize("B,M,N,K,d1", [
+    (10240, 88, 64, 88, 10), (24, 80, 64, 88, 12), (100, 88, 64, 88, 10),     # tests/unittest/ops/test_bmm_permute.py:109-117
+    (768, 384, 384, 64, 12),                                                   # attention scores of BERT-base, per head
+    (6, 33, 20, 24, 3), (4, 1, 8, 8, 4), (5, 130, 72, 40, 1),
+])
+def test_bmm_rcr_permute(B, M, N, K, d1):
+    print(f"case bmm_rcr_permute B={B} M={M} N={N} K={K} d1={d1}", flush=True)
+    q, k = _rand((B, M, K), torch.float16, 1), _rand((B, N, K), torch.float16, 2, K ** -0.5)
+    qd, kd = q.cuda(), k.cuda()
+    got = eager.bmm_rcr_permute(qd, kd, (d1,))
+    plain = eager.bmm_rcr(qd, kd)
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (B // d1, M, d1, N)
+    # the permutation moves elements of the plain result, bit for bit (same heuristic instance: same shape)
+    assert torch.equal(got.cpu(), plain.cpu().reshape(B // d1, d1, M, N).permute(0, 2, 1, 3))
+    if B * M * N <= 1 << 24:
+        want = oracle.torch_bmm_rcr_permute(q, k, d1).half().float()
+        torch.testing.assert_close(got.cpu().float(), want, atol=1e-2, rtol=1e-2)
+
+
+def test_bmm_rcr_permute_every_instance_and_errors():
+    B, M, N, K, d1 = 12, 200, 136, 72, 4
+    q, k = _rand((B, M, K), torch.float16, 3).cuda(), _rand((B, N, K), torch.float16, 4, K ** -0.5).cuda()
+    lib = _kernels.load()
+    for algo, name in enumerate(_kernels.gemm_algo_names(0, 0)):
+        if not lib.aitamd_gemm_algo_supported(0, 0, algo, M, N, K, K, K, 16):
+            continue
+        print(f"case bmm_rcr_permute instance={name}", flush=True)
+        got = eager.bmm_rcr_permute(q, k, (d1,), algo=algo)
+        plain = eager.bmm_rcr(q, k, algo=algo)
+        torch.cuda.synchronize()
+        assert torch.equal(got, plain.reshape(B // d1, d1, M, N).permute(0, 2, 1, 3))
+    with pytest.raises(ValueError, match="multiple"):
+        eager.bmm_rcr_permute(q, k, (5,))
+    out = torch.empty(B * M * N, dtype=torch.float16, device="cuda")
+    assert lib.aitamd_bmm_rcr_permute(0, -1, q.data_ptr(), k.data_ptr(), out.data_ptr(), B, M, N, K, K, K, M * K,
+                                      N * K, 5, None) != 0
+    assert b"multiple" in lib.aitamd_last_error()

@@ -276,3 +276,14 @@ def test_attention_block_matches_torch_nn_multiheadattention(causal):
         got = oracle.torch_multihead_attention(x, mha.in_proj_weight, mha.in_proj_bias, mha.out_proj.weight,
                                                mha.out_proj.bias, res, H, causal)
     assert torch.allclose(got, want + res.reshape(B, S, D), atol=1e-5)
+
+
+def test_bmm_rcr_permute_places_each_batch_as_a_head():
+    """out[g, m, h, n] must be (Q[g*d1 + h] @ K[g*d1 + h]^T)[m, n]: brute force over the batch index."""
+    B, M, N, K, d1 = 6, 5, 7, 4, 3
+    q, k = _rand((B, M, K), seed=1), _rand((B, N, K), seed=2)
+    out = oracle.torch_bmm_rcr_permute(q, k, d1)
+    assert tuple(out.shape) == (B // d1, M, d1, N)
+    for b in range(B):
+        want = q[b].float() @ k[b].float().T
+        assert torch.allclose(out[b // d1, :, b % d1, :], want, atol=1e-5)
