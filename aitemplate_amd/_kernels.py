@@ -50,7 +50,9 @@ DTYPE_ID = {"float16": 0, "bfloat16": 1}
 # On ROCm the reference lowers layout "20314" like "m3n2" (gemm_rcr_bias_permute.py:66-72 of
 # python/aitemplate/compiler/ops/gemm_universal/).
 PERMUTE_M2N3, PERMUTE_M3N2 = 1, 2
-BMM_PERMUTE_OPS = ("bmm_rcr_permute",)  # epilogue 0, launched through aitamd_bmm_rcr_permute
+LAYOUT_ID = {"rcr": 0, "rrr": 1, "ccr": 2, "crr": 3}
+# plain-epilogue ops launched through aitamd_bmm / aitamd_bmm_rcr_permute
+LAYOUT_OPS = ("bmm_rcr_permute", "bmm_rrr", "bmm_rrr_permute", "bmm_ccr", "bmm_crr", "gemm_rrr")
 PERMUTE_OPS = {
     "gemm_rcr_permute_m2n3": (0, PERMUTE_M2N3),
     "gemm_rcr_bias_permute_m2n3": (1, PERMUTE_M2N3),
@@ -70,6 +72,9 @@ EXPORTED_SYMBOLS = [
     "aitamd_gemm_rcr",
     "aitamd_gemm_rcr_permute",
     "aitamd_bmm_rcr_permute",
+    "aitamd_bmm",
+    "aitamd_gemm_algo_supported_layout",
+    "aitamd_gemm_heuristic_algo_layout",
     "aitamd_bmm_rcr",
     "aitamd_bmm_softmax_bmm_permute",
 ]
@@ -115,6 +120,12 @@ def load() -> ctypes.CDLL:
         lib.aitamd_gemm_rcr_permute.argtypes = [i32, i32, i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, i64, i64, i64, vp]
         lib.aitamd_bmm_rcr_permute.restype = i32
         lib.aitamd_bmm_rcr_permute.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
+        lib.aitamd_bmm.restype = i32
+        lib.aitamd_bmm.argtypes = [i32, i32, i32, vp, vp, vp] + [i64] * 11 + [vp]
+        lib.aitamd_gemm_algo_supported_layout.restype = i32
+        lib.aitamd_gemm_algo_supported_layout.argtypes = [i32, i32, i32, i32, i64, i64, i64, i64, i64, i32]
+        lib.aitamd_gemm_heuristic_algo_layout.restype = i32
+        lib.aitamd_gemm_heuristic_algo_layout.argtypes = [i32, i32, i32, i64, i64, i64, i64, i64, i64, i32]
         lib.aitamd_bmm_rcr.restype = i32
         lib.aitamd_bmm_rcr.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
         lib.aitamd_bmm_softmax_bmm_permute.restype = i32

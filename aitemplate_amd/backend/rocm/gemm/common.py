@@ -36,7 +36,7 @@ EXTRA_PTRS = {0: [], 1: ["bias_ptr"]}
 def epilogue_id(op_name: str) -> int:
     if op_name in _kernels.PERMUTE_OPS:
         return _kernels.PERMUTE_OPS[op_name][0]
-    if op_name in _kernels.BMM_PERMUTE_OPS:
+    if op_name in _kernels.LAYOUT_OPS:
         return 0
     return _kernels.EPILOGUE_OF_OP[op_name]
 

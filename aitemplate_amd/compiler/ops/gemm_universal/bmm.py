@@ -1,8 +1,9 @@
-"""Batched GEMM: the bmm base class, bmm_rcr and bmm_rcr_permute.
+"""Batched GEMM: the bmm base class, the four operand layouts with a row-major result (rcr, rrr, ccr, crr)
+and the *_permute forms of rcr and rrr.
 
-Counterparts: python/aitemplate/compiler/ops/gemm_universal/bmm.py:69-119 (base, batch
-broadcast rules) and bmm_xxx.py:22-150,261-278 (layout bookkeeping; only the r-c-r
-layout exists on this backend)."""
+Counterparts: python/aitemplate/compiler/ops/gemm_universal/bmm.py:69-119 (base, batch broadcast rules),
+bmm_xxx.py:22-150,204-278 (layout bookkeeping), bmm_rcr_permute.py, bmm_rrr_permute.py.  The layouts with a
+column-major result (bmm_xxc) exist on CUDA only in the reference."""
 from ...base import IntImm, Tensor
 from ...dtype import is_same_dtype
 from ...tensor_accessor import TensorAccessor
@@ -111,3 +112,80 @@ class bmm_rcr_permute(bmm_rcr):
 
     def _get_op_attributes(self):
         return {"layout": self._attrs["layout"].split("_")[-1], "shape": self._attrs["shape"]}
+
+
+def _layout_class(name: str, a_col: bool, b_row: bool, doc: str):
+    """A [B, M, K] (or [B, K, M] when a_col) times B [B, N, K] (or [B, K, N] when b_row) -> [B, M, N]."""
+
+    class _bmm_layout(bmm):
+        __doc__ = doc
+
+        def __init__(self):
+            super().__init__()
+            self._attrs["op"] = name
+
+            def cal_align_ab(m, n, k):
+                # the contiguous dim of each operand bounds the load width (bmm_xxx.py:36-43)
+                return common.default_align_ab(m if a_col else k, n if b_row else k,
+                                               self._attrs["inputs"][0].dtype())
+
+            self._attrs["f_ab_alignment"] = cal_align_ab
+
+        def _mk(self, a: Tensor, b: Tensor):
+            a_shape, b_shape = a.shape(), b.shape()
+            m, ka = (a_shape[-1], a_shape[-2]) if a_col else (a_shape[-2], a_shape[-1])
+            n, kb = (b_shape[-1], b_shape[-2]) if b_row else (b_shape[-2], b_shape[-1])
+            return m, n, ka, kb
+
+        def _infer_shapes(self, a: Tensor, b: Tensor):
+            m, n, ka, kb = self._mk(a, b)
+            if ka != kb:
+                raise RuntimeError(f"{name} operand A and B should have the same K dim! A: {a.shape()}, B: {b.shape()}")
+            return [self._get_batch_size(a, b), m, n]
+
+        def _extract_dims(self, for_profiling: bool = False):
+            S = common.Source
+            a_shapes = common.extract_shape_from_accessor(self._attrs, S.INPUT, 0)
+            b_shapes = common.extract_shape_from_accessor(self._attrs, S.INPUT, 1)
+            out_shapes = common.extract_shape_from_accessor(self._attrs, S.OUTPUT, 0)
+            b_dim = common.create_input_batch_diminfo([a_shapes, b_shapes], [0, 0], out_shapes[0])
+            b_dim.append(common.DimInfo(S.OUTPUT, tensor_idx=0, dim_idx=0))
+            ra, rb = len(a_shapes), len(b_shapes)
+            a_m, a_k = (ra - 1, ra - 2) if a_col else (ra - 2, ra - 1)
+            b_n, b_k = (rb - 1, rb - 2) if b_row else (rb - 2, rb - 1)
+            return {
+                "B": b_dim,
+                "M": [common.DimInfo(S.INPUT, tensor_idx=0, dim_idx=a_m), common.DimInfo(S.OUTPUT, tensor_idx=0, dim_idx=1)],
+                "N": [common.DimInfo(S.INPUT, tensor_idx=1, dim_idx=b_n), common.DimInfo(S.OUTPUT, tensor_idx=0, dim_idx=2)],
+                "K": [common.DimInfo(S.INPUT, tensor_idx=0, dim_idx=a_k), common.DimInfo(S.INPUT, tensor_idx=1, dim_idx=b_k)],
+            }
+
+        def _align_ab(self, a: Tensor, b: Tensor):
+            _, _, ka, kb = self._mk(a, b)
+            if not isinstance(ka, IntImm) or not isinstance(kb, IntImm):
+                raise RuntimeError(f"K must be static! A: {a.shape()}, B: {b.shape()}")
+            return a, b
+
+    _bmm_layout.__name__ = _bmm_layout.__qualname__ = name
+    return _bmm_layout
+
+
+bmm_rrr = _layout_class("bmm_rrr", False, True, "C[b] = A[b] @ B[b] with A [B, M, K], B [B, K, N] (torch.bmm(A, B)).")
+bmm_ccr = _layout_class("bmm_ccr", True, False,
+                        "C[b] = A[b]^T @ B[b]^T with A [B, K, M], B [B, N, K].")
+bmm_crr = _layout_class("bmm_crr", True, True, "C[b] = A[b]^T @ B[b] with A [B, K, M], B [B, K, N].")
+
+
+class bmm_rrr_permute(bmm_rrr):
+    """bmm_rrr whose [B, M, N] result is stored as [B // d1, M, d1, N] with shape = (d1,) (layout "0213").
+    Counterpart of python/aitemplate/compiler/ops/gemm_universal/bmm_rrr_permute.py."""
+
+    def __init__(self, shape, layout="0213"):
+        super().__init__()
+        self._attrs["op"] = "bmm_rrr_permute"
+        self._attrs["shape"] = tuple(int(v) for v in shape)
+        self._attrs["layout"] = "Permute4DBMM_{}".format(layout)
+        self._attrs["permute_shape"] = "_".join(map(str, shape))
+
+    __call__ = bmm_rcr_permute.__call__
+    _get_op_attributes = bmm_rcr_permute._get_op_attributes

@@ -358,10 +358,19 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           for (int e = 0; e < 16; ++e) text = fmaxf(text, s[e]);
         }
         text = neg_scale ? min_across_halves(text) : max_across_halves(text);
-        const float m_new = neg_scale ? fminf(m_run, text) : fmaxf(m_run, text);
-        const float m_safe = __builtin_isinf(m_new) ? 0.0f : m_new;  // every key so far masked
+        const float m_cand = neg_scale ? fminf(m_run, text) : fmaxf(m_run, text);
+        // The reference point of the exponent moves only when the row extremum has grown by more than
+        // kLazyLog2 binary orders since it was last taken: until then p = exp2(s c - m c) may exceed 1 (by at
+        // most 2^kLazyLog2, harmless in fp32 sums and in the fp16 / bf16 probabilities) and the accumulators
+        // need no rescaling.  With random scores some row of a wave sets a new maximum in most blocks, so
+        // rescaling on every change costs 2 multiplies per score; this way it is rare.
+        constexpr float kLazyLog2 = 8.0f;
         const float c = p.scale_log2e;
-        const float alpha = __builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m_safe) * c);
+        const float drift = (m_run - m_cand) * c;  // <= 0; -inf (or NaN for inf - inf) on the first live block
+        const bool move = !(drift >= -kLazyLog2);
+        const float m_new = move ? m_cand : m_run;
+        const float m_safe = __builtin_isinf(m_new) ? 0.0f : m_new;  // every key so far masked
+        const float alpha = !move ? 1.0f : (__builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f(drift));
         const float mc = -m_safe * c;
         float psum = 0.0f;
         if (need_mask) {

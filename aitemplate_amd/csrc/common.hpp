@@ -61,6 +61,28 @@ struct ElemTraits<bf16> {
   static AITAMD_DEVICE bf16 from_float(float v) { return (bf16)v; }
 };
 
+// LDS transpose read: 4 x 16-bit per lane, gathered across the 16 lanes of a block
+AITAMD_DEVICE f16x4 tr_read16(const f16* p) {
+  typedef __fp16 raw4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+  const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((__attribute__((address_space(3))) raw4*)p);
+  return __builtin_bit_cast(f16x4, r);
+}
+AITAMD_DEVICE bf16x4 tr_read16(const bf16* p) {
+  typedef __bf16 raw4 __attribute__((__vector_size__(4 * sizeof(__bf16))));
+  const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) raw4*)p);
+  return __builtin_bit_cast(bf16x4, r);
+}
+template <class T>
+AITAMD_DEVICE typename ElemTraits<T>::vec8 join_halves(typename ElemTraits<T>::vec4 lo, typename ElemTraits<T>::vec4 hi) {
+  typename ElemTraits<T>::vec8 v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    v[j] = lo[j];
+    v[4 + j] = hi[j];
+  }
+  return v;
+}
+
 // ---------------------------------------------------------------------------
 // Raw buffer resources.  Loads whose byte offset is >= num_records return 0,
 // which is how every M/N/K tail is zero-filled without branches.

@@ -19,6 +19,7 @@ struct GemmAlgo {
   int lds_bytes;
   int wgs_per_cu;  // workgroups of this instance one CU holds at once
   int direct_lds;  // 0: register-staged loads, 1: direct-to-LDS ring, 2: persistent direct-to-LDS ring
+  int layouts;     // bit L set: a kernel for operand layout L exists (0 rcr, 1 rrr, 2 ccr, 3 crr)
   hipError_t (*launch)(const GemmParams& p, hipStream_t stream);
 };
 

@@ -34,19 +34,33 @@ using Epi = Epilogue<AITAMD_EPI>;
 // Kernels with the permuted store exist for the two epilogues the permuting ops use.
 constexpr bool kHasPermutedStore = AITAMD_EPI == kEpiNone || AITAMD_EPI == kEpiBias;
 
-template <class Tile, bool PERM>
+// Kernels for operands that are not K-contiguous (layouts rrr, ccr, crr) exist for the plain epilogue, on the
+// direct-to-LDS tiles whose edges allow it.
+constexpr bool kHasLayouts = AITAMD_EPI == kEpiNone;
+
+template <class Tile, bool PERM, int LAYOUT>
 struct KernelOf {
   static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi, PERM>;
 };
-template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, bool PERM>
-struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, PERM> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, bool PERM, int LAYOUT>
+struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, PERM, LAYOUT> {
   static constexpr auto value =
-      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, Epi, PERM>;
+      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, Epi, PERM, LAYOUT>;
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int NS, bool PERM>
-struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS>, PERM> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, bool PERM, int LAYOUT>
+struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS>, PERM, LAYOUT> {
   static constexpr auto value = gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS>, Epi, PERM>;
+};
+// bit L set: the tile has a kernel for layout L (bit 0, rcr, always)
+template <class Tile>
+struct LayoutMask {
+  static constexpr int value = 1;
+};
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
+struct LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>> {
+  static constexpr int value =
+      (kHasLayouts && GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kTransposable) ? 0xf : 1;
 };
 template <class Tile>
 struct IsPersistent {
@@ -68,9 +82,9 @@ inline int device_cus(int dev) {
   return v;
 }
 
-template <class Tile, bool PERM>
+template <class Tile, bool PERM, int LAYOUT = 0>
 hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
-  auto kernel = KernelOf<Tile, PERM>::value;
+  auto kernel = KernelOf<Tile, PERM, LAYOUT>::value;
   // LDS above 64 KiB has to be opted into once per device.
   static std::once_flag once[kMaxDevices];
   int dev = 0;
@@ -109,6 +123,17 @@ hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
 
 template <class Tile>
 hipError_t launch_tile(const GemmParams& p, hipStream_t stream) {
+  if (p.layout != 0) {
+    if constexpr (LayoutMask<Tile>::value == 0xf) {
+      if (p.perm_on) return hipErrorInvalidValue;
+      switch (p.layout) {
+        case 1: return launch_kernel<Tile, false, 1>(p, stream);
+        case 2: return launch_kernel<Tile, false, 2>(p, stream);
+        case 3: return launch_kernel<Tile, false, 3>(p, stream);
+      }
+    }
+    return hipErrorInvalidValue;
+  }
   if (p.perm_on) {
     if constexpr (kHasPermutedStore) return launch_kernel<Tile, true>(p, stream);
     return hipErrorInvalidValue;
@@ -143,7 +168,7 @@ const GemmAlgo kAlgos[] = {
    BM, BN, BK, GemmTile<BM, BN, BK, WM, WN, KV>::NT, KV, GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes, \
    staged_wgs_per_cu(BM, BN, GemmTile<BM, BN, BK, WM, WN, KV>::NT,                                  \
                      GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes),                                  \
-   0, &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
+   0, 1, &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
 #define AITAMD_GEMM_TILE_DMA(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX)                                 \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
    "_c" #AUX,                                                                                              \
@@ -151,11 +176,12 @@ const GemmAlgo kAlgos[] = {
    GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kLdsBytes,                                     \
    dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::NT, OCC,                        \
                   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kLdsBytes),                      \
-   1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>},
+   1, LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>::value,                            \
+   &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>},
 #define AITAMD_GEMM_TILE_PERSIST(BM, BN, BK, WM, WN, NS)                                                  \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_persist" #NS,                      \
    BM, BN, BK, GemmTilePersist<BM, BN, BK, WM, WN, NS>::NT, 8, GemmTilePersist<BM, BN, BK, WM, WN, NS>::kLdsBytes, \
-   1, 2, &launch_tile<GemmTilePersist<BM, BN, BK, WM, WN, NS>>},
+   1, 2, 1, &launch_tile<GemmTilePersist<BM, BN, BK, WM, WN, NS>>},
 #include "gemm_tiles.inc"
 #undef AITAMD_GEMM_TILE
 #undef AITAMD_GEMM_TILE_DMA

@@ -50,6 +50,9 @@ struct GemmParams {
   // bmm_rcr_permute with batch_inner = d1, sc = N, sc_outer = M * d1 * N and ldc = d1 * N.
   int32_t batch_inner;
   int64_t sc_outer;
+  // operand layout: 0 rcr (A [M, K], B [N, K]), 1 rrr (B [K, N]), 2 ccr (A [K, M]), 3 crr (both); lda / ldb
+  // are the row pitches of the matrices as stored
+  int32_t layout;
 };
 
 AITAMD_DEVICE int64_t out_batch_offset(const GemmParams& p, int batch) {

@@ -53,6 +53,9 @@ struct GemmTileDma {
   static constexpr int EPI_BYTES = NW * MT * EPI_PITCH * 4;
   static constexpr int MAIN_BYTES = NS * STAGE_ELEMS * 2;
   static constexpr int kLdsBytes = MAIN_BYTES > EPI_BYTES ? MAIN_BYTES : EPI_BYTES;
+  // operands that are not K-contiguous need whole k-rows per 1 KiB wave-load and at least 8 chunks per row
+  static constexpr bool kTransposable = MT == 32 && (BM == 64 || BM == 128 || BM == 256) &&
+      (BN == 64 || BN == 128 || BN == 256);
   static_assert(MT == 32 || MT == 16, "MFMA tile is 32x32 or 16x16");
   static_assert(WTM % MT == 0 && WTN % MT == 0, "wave tile must be whole MFMA tiles");
   static_assert(BM % ROWS_PER_LOAD == 0 && BN % ROWS_PER_LOAD == 0, "slab rows must fill whole wave-loads");
@@ -131,10 +134,22 @@ AITAMD_DEVICE void sched_step() {
   sched_spread_vmem<VM, REST, PER>();
 }
 
-template <class T, class Tile, class Epi, bool PERM = false>
+// LAYOUT selects how the operands lie in memory (the result is always row-major):
+//   0 "rcr": A [M, K], B [N, K]  - both K-contiguous, the native form of the MFMA operands
+//   1 "rrr": A [M, K], B [K, N]      2 "ccr": A [K, M], B [N, K]      3 "crr": A [K, M], B [K, N]
+// An operand that is not K-contiguous is copied to LDS as it lies in memory (k-rows of BM or BN elements,
+// 16-byte chunks XOR-swizzled by 2 * (k % 4) so that four consecutive k-rows fall into four different
+// 32-byte bank groups) and its fragments are gathered with the transposing LDS read: per 16 lanes, lane
+// 4 i + e receives element e of the four 8-byte rows i, i + 4, i + 8, i + 12 addressed by the 16 lanes, so
+// when lane r points at (k-row r / 4, elements 4 (r % 4) .. + 4) lane d ends up with one element column d
+// of four consecutive k-rows: two such reads give the 8 k-values of an MFMA operand.
+template <class T, class Tile, class Epi, bool PERM = false, int LAYOUT = 0>
 __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const GemmParams p) {
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
+  using vec4 = typename Tr::vec4;
+  constexpr bool A_T = (LAYOUT & 2) != 0, B_T = (LAYOUT & 1) != 0;
+  static_assert(LAYOUT == 0 || Tile::kTransposable, "this tile has no transposed-operand form");
   using Mfma = MfmaOp<T, Tile::MT>;
   using acc_t = typename Mfma::acc_t;
   constexpr int BM = Tile::BM, BN = Tile::BN, BK = Tile::BK, NS = Tile::NS;
@@ -169,15 +184,29 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
   // wave-load j (j = wave + i * NW) fills 1 KiB block j of the slab; blocks
   // [0, A_LOADS) belong to A, the rest to B.  j is wave-uniform.
   uint32_t l_off[L_IT];
-  int l_chunk_k[L_IT];
+  int l_chunk_k[L_IT];      // k offset inside the slab of the lane's chunk (its k-row for a transposed operand)
+  uint32_t l_kbytes[L_IT];  // bytes one step in k moves the lane's source address
 #pragma unroll
   for (int i = 0; i < L_IT; ++i) {
     const int j = wave + i * Tile::NW;
     const bool is_a = j < Tile::A_LOADS;
-    const int row = (is_a ? j : j - Tile::A_LOADS) * Tile::ROWS_PER_LOAD + l_row;
-    const int chunk = l_slot ^ ((row / Tile::RPW) % Tile::CPR);
-    l_off[i] = (uint32_t)(((int64_t)row * (is_a ? p.lda : p.ldb) + chunk * 8) * 2);
-    l_chunk_k[i] = chunk * 8;
+    const int64_t ld = is_a ? p.lda : p.ldb;
+    if ((is_a && A_T) || (!is_a && B_T)) {
+      // 1 KiB of the operand's slab = 512 / BX whole k-rows of BX elements
+      const int bx = is_a ? BM : BN;
+      const int cpr = bx / 8;
+      const int k_row = (is_a ? j : j - Tile::A_LOADS) * (512 / bx) + lane / cpr;
+      const int chunk = (lane % cpr) ^ (2 * (k_row & 3));
+      l_off[i] = (uint32_t)(((int64_t)k_row * ld + chunk * 8) * 2);
+      l_chunk_k[i] = k_row;
+      l_kbytes[i] = (uint32_t)(ld * 2);
+    } else {
+      const int row = (is_a ? j : j - Tile::A_LOADS) * Tile::ROWS_PER_LOAD + l_row;
+      const int chunk = l_slot ^ ((row / Tile::RPW) % Tile::CPR);
+      l_off[i] = (uint32_t)(((int64_t)row * ld + chunk * 8) * 2);
+      l_chunk_k[i] = chunk * 8;
+      l_kbytes[i] = 2;
+    }
   }
 
   int a_rd[KK], b_rd[KK];
@@ -186,14 +215,36 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     a_rd[kk] = dma_lds_chunk_elem<Tile>(wm * Tile::WTM + fr, kk * QN + fq);
     b_rd[kk] = BM * BK + dma_lds_chunk_elem<Tile>(wn * Tile::WTN + fr, kk * QN + fq);
   }
+  // transposed operands: lane r of a 16-lane block addresses k-row (r / 4) and the 8-byte piece (r % 4) of
+  // the block's 16 element columns; blocks 0 / 1 take the lower / upper 16 columns of a 32-wide MFMA
+  // operand, blocks 2 / 3 the second 8 k-values (lane / 32, as for the K-contiguous operands)
+  const int t_r = lane & 15;
+  const int t_swz = 2 * ((t_r >> 2) & 3);
+  const int t_piece = ((lane >> 4) & 1) * 2 + ((t_r & 3) >> 1);  // 16-byte chunk inside the 32 columns
+  int at_col[A_T ? MI : 1], bt_col[B_T ? NI : 1];
+  if constexpr (A_T) {
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+      at_col[mi] = (((wm * Tile::WTM / 8 + mi * 4 + t_piece) ^ t_swz) << 3) + (t_r & 1) * 4 +
+          (fq * 8 + (t_r >> 2)) * BM;
+  }
+  if constexpr (B_T) {
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+      bt_col[ni] = BM * BK + (((wn * Tile::WTN / 8 + ni * 4 + t_piece) ^ t_swz) << 3) + (t_r & 1) * 4 +
+          (fq * 8 + (t_r >> 2)) * BN;
+  }
 
   const int k_tiles = (p.K + BK - 1) / BK;
 
   {
-    const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)batch * p.sa + (int64_t)m0 * p.lda;
-    const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)batch * p.sb + (int64_t)n0 * p.ldb;
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ab, clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2));
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
+    // a transposed operand starts at its first column of the tile and ends with the tile's columns of row K-1
+    const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)batch * p.sa + (A_T ? (int64_t)m0 : (int64_t)m0 * p.lda);
+    const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)batch * p.sb + (B_T ? (int64_t)n0 : (int64_t)n0 * p.ldb);
+    const int64_t bytes_a = A_T ? (((int64_t)p.K - 1) * p.lda + rows_a) * 2 : (((int64_t)rows_a - 1) * p.lda + p.K) * 2;
+    const int64_t bytes_b = B_T ? (((int64_t)p.K - 1) * p.ldb + rows_b) * 2 : (((int64_t)rows_b - 1) * p.ldb + p.K) * 2;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ab, clamp_records(bytes_a));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bb, clamp_records(bytes_b));
 
     // Issue the wave-loads of K-slab `kt` into ring slot `stage`.  Slabs past
     // the end of K are still issued (every chunk out of range -> zero fill) so
@@ -205,7 +256,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
       for (int i = 0; i < L_IT; ++i) {
         if (i < i0 || i >= i1) continue;
         const int j = wave + i * Tile::NW;
-        const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + (uint32_t)(k0 * 2) : kOobOffset;
+        const uint32_t step = (A_T || B_T) ? (uint32_t)k0 * l_kbytes[i] : (uint32_t)(k0 * 2);
+        const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + step : kOobOffset;
         T* dst = sbase + j * 512;  // 1 KiB = 512 elements per wave-load; A blocks then B blocks
         if (j < Tile::A_LOADS)
           __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)dst, 16, off, 0, 0, AUX);
@@ -214,6 +266,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
       }
     };
 
+    constexpr int kFragReads = MI * (A_T ? 2 : 1) + NI * (B_T ? 2 : 1);  // LDS reads per MFMA step
     acc_t acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -237,9 +290,23 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
 
     auto load_frags = [&](const T* st, int kk, vec8* af, vec8* bf) {
 #pragma unroll
-      for (int mi = 0; mi < MI; ++mi) af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[kk] + mi * MT * BK);
+      for (int mi = 0; mi < MI; ++mi) {
+        if constexpr (A_T) {
+          const T* at = st + at_col[mi] + kk * Tile::KSTEP * BM;
+          af[mi] = join_halves<T>(tr_read16(at), tr_read16(at + 4 * BM));
+        } else {
+          af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[kk] + mi * MT * BK);
+        }
+      }
 #pragma unroll
-      for (int ni = 0; ni < NI; ++ni) bf[ni] = *reinterpret_cast<const vec8*>(st + b_rd[kk] + ni * MT * BK);
+      for (int ni = 0; ni < NI; ++ni) {
+        if constexpr (B_T) {
+          const T* bt = st + bt_col[ni] + kk * Tile::KSTEP * BN;
+          bf[ni] = join_halves<T>(tr_read16(bt), tr_read16(bt + 4 * BN));
+        } else {
+          bf[ni] = *reinterpret_cast<const vec8*>(st + b_rd[kk] + ni * MT * BK);
+        }
+      }
     };
     // operands swapped: the MFMA produces the transposed tile, so a lane holds
     // 4 consecutive output columns of one row
@@ -267,7 +334,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
           if (kk + 1 < KK) load_frags(cur, kk + 1, af[nb], bf[nb]);
           mfmas(af[cb], bf[cb]);
           if (kk + 1 < KK)
-            sched_step<MI * NI, MI + NI, L_PER>();
+            sched_step<MI * NI, kFragReads, L_PER>();
           else
             sched_step<MI * NI, 0, L_PER>();
         }
@@ -295,7 +362,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
               issue_loads(kt + NS - 2, (kt + NS - 2) % NS, i0, i1);
               load_frags(cur, kk + 1, af[nb], bf[nb]);
               mfmas(af[cb], bf[cb]);
-              sched_step<MI * NI, MI + NI, L_PER>();
+              sched_step<MI * NI, kFragReads, L_PER>();
             } else {
               // slab kt+1 has landed once at most (NS-3) younger slabs are in flight;
               // past the barrier nobody reads slab kt-1 any more, so its ring slot
@@ -307,7 +374,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
               issue_loads(kt + NS - 1, (kt + NS - 1) % NS, 0, i1);
               load_frags(smem + ((kt + 1) % NS) * Tile::STAGE_ELEMS, 0, af[nb], bf[nb]);
               mfmas(af[cb], bf[cb]);
-              sched_step<MI * NI, MI + NI, L_P0>();
+              sched_step<MI * NI, kFragReads, L_P0>();
             }
           }
         }

@@ -140,6 +140,7 @@ struct OperandSet {
 struct PermuteSpec {
   int layout = 0;
   int64_t g[3] = {1, 1, 1};
+  int operands = 0;  // operand layout of the batched launcher: AITAMD_LAYOUT_*
 };
 
 // permuting op name -> base op (which names the epilogue) and layout id; false when `op` does not permute
@@ -212,6 +213,11 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
     if (perm.layout && !batched)
       return aitamd_gemm_rcr_permute(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.c.p, M, N, K, K, K, perm.layout,
                                      perm.g[0], perm.g[1], perm.g[2], stream);
+    if (batched && perm.operands != AITAMD_LAYOUT_RCR) {
+      const int64_t lda = (perm.operands & 2) ? M : K, ldb = (perm.operands & 1) ? N : K;
+      return aitamd_bmm(perm.operands, dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, lda, ldb, N, M * K, N * K, M * N,
+                        perm.layout ? perm.g[0] : 0, stream);
+    }
     if (batched && perm.layout)  // bmm_rcr_permute: perm.g[0] = d1
       return aitamd_bmm_rcr_permute(dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, K, K, M * K, N * K, perm.g[0], stream);
     if (batched)
@@ -227,7 +233,12 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
       const bool numeric = only[0] >= '0' && only[0] <= '9';
       if (numeric ? atoi(only) != algo : strcmp(only, name) != 0) continue;
     }
-    if (!aitamd_gemm_algo_supported(epi, dtype, algo, M, N, K, K, K, 16)) continue;
+    if (perm.operands != AITAMD_LAYOUT_RCR) {
+      const int64_t lda = (perm.operands & 2) ? M : K, ldb = (perm.operands & 1) ? N : K;
+      if (!aitamd_gemm_algo_supported_layout(epi, dtype, perm.operands, algo, M, N, K, lda, ldb, 16)) continue;
+    } else if (!aitamd_gemm_algo_supported(epi, dtype, algo, M, N, K, K, K, 16)) {
+      continue;
+    }
     bool ok = true;
     for (int i = 0; i < warmup && ok; ++i) ok = launch(algo, pool[i % sets]) == 0;
     if (!ok) {
@@ -301,7 +312,7 @@ int profile_attention(int dtype, int64_t B, int64_t M, int64_t N, int64_t K, int
 
 int main(int argc, char** argv) {
   if (argc < 4) {
-    fprintf(stderr, "usage: %s gemm|gemm_permute|bmm|bmm_permute|attn <op> <dtype> dims...\n", argv[0]);
+    fprintf(stderr, "usage: %s gemm|gemm_permute|gemm_layout|bmm|bmm_permute|bmm_layout|attn <op> <dtype> dims...\n", argv[0]);
     return 2;
   }
   const std::string kind = argv[1];
@@ -336,6 +347,21 @@ int main(int argc, char** argv) {
     perm.layout = 1;
     perm.g[0] = d[4];
     return profile_gemm_like("bmm_rcr", dtype, d[0], d[1], d[2], d[3], true, perm);
+  }
+  if (kind == "bmm_layout" || kind == "gemm_layout") {  // bmm_rrr[_permute] | bmm_ccr | bmm_crr: B M N K [d1]; gemm_rrr: M N K
+    const bool batched = kind == "bmm_layout";
+    const size_t need = batched ? 4 : 3;
+    const size_t lay_at = op.find('_');
+    if (d.size() < need || lay_at == std::string::npos || op.size() < lay_at + 4) return 2;
+    PermuteSpec perm;
+    perm.operands = (op[lay_at + 1] == 'c' ? 2 : 0) | (op[lay_at + 2] == 'r' ? 1 : 0);
+    if (op.size() > 8 && op.compare(op.size() - 8, 8, "_permute") == 0) {
+      if (d.size() < need + 1) return 2;
+      perm.layout = 1;
+      perm.g[0] = d[need];
+    }
+    if (batched) return profile_gemm_like("bmm_rcr", dtype, d[0], d[1], d[2], d[3], true, perm);
+    return profile_gemm_like("bmm_rcr", dtype, 1, d[0], d[1], d[2], true, perm);
   }
   if (kind == "attn") {
     if (d.size() < 6) return 2;

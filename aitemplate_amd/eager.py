@@ -157,6 +157,42 @@ def bmm_rcr(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None
     return out
 
 
+def bmm(layout: str, a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None, d1: int = 0,
+        algo: int = -1) -> torch.Tensor:
+    """Batched GEMM for the operand layouts "rcr", "rrr", "ccr", "crr" of the reference
+    (python/aitemplate/compiler/ops/gemm_universal/bmm_xxx.py): first letter r = A is [B, M, K], c = A is
+    [B, K, M]; second letter r = B is [B, K, N], c = B is [B, N, K]; the result is [B, M, N], or
+    [B // d1, M, d1, N] when d1 > 0 (the *_permute ops).  2-D or batch-1 operands broadcast."""
+    lib = _kernels.load()
+    lay = _kernels.LAYOUT_ID[layout]
+    dtype = a.dtype
+    for t, n in ((a, "a"), (b, "b"), (out, "out")):
+        _check(t, n, dtype)
+    a3 = a if a.dim() == 3 else a.unsqueeze(0)
+    b3 = b if b.dim() == 3 else b.unsqueeze(0)
+    if not (a3.is_contiguous() and b3.is_contiguous()):
+        raise ValueError("bmm operands must be contiguous")
+    B = max(a3.shape[0], b3.shape[0])
+    if a3.shape[0] not in (1, B) or b3.shape[0] not in (1, B):
+        raise ValueError("batch sizes must match or be 1")
+    M, K = (a3.shape[2], a3.shape[1]) if lay & 2 else (a3.shape[1], a3.shape[2])
+    N, Kb = (b3.shape[2], b3.shape[1]) if lay & 1 else (b3.shape[1], b3.shape[2])
+    if Kb != K:
+        raise ValueError("K mismatch")
+    if d1 and (d1 < 0 or B % d1):
+        raise ValueError(f"batch {B} is not a multiple of d1 = {d1}")
+    if out is None:
+        out = torch.empty((B // d1, M, d1, N) if d1 else (B, M, N), dtype=dtype, device=a.device)
+    elif not out.is_contiguous() or out.numel() != B * M * N:
+        raise ValueError("out must be contiguous with B*M*N elements")
+    sa = 0 if (a3.shape[0] == 1 and B > 1) else M * K
+    sb = 0 if (b3.shape[0] == 1 and B > 1) else N * K
+    rc = lib.aitamd_bmm(lay, _TORCH_DTYPE_ID[dtype], algo, _p(a3), _p(b3), _p(out), B, M, N, K, a3.shape[2],
+                        b3.shape[2], N, sa, sb, M * N, d1, _stream_ptr())
+    _kernels.check(rc, f"bmm_{layout}")
+    return out
+
+
 def bmm_rcr_permute(a: torch.Tensor, b: torch.Tensor, shape, out: Optional[torch.Tensor] = None,
                     algo: int = -1) -> torch.Tensor:
     """bmm_rcr stored as [B // d1, M, d1, N] with shape = (d1,)

@@ -138,6 +138,28 @@ AITAMD_API int aitamd_bmm_rcr(int dtype, int algo,
                               int64_t stride_a, int64_t stride_b, int64_t stride_c,
                               void* stream);
 
+/* Batched GEMM for the reference's other operand layouts; the result is row-major [B, M, N] in all of them.
+ *   AITAMD_LAYOUT_RCR: A [B, M, K], B [B, N, K]     AITAMD_LAYOUT_RRR: A [B, M, K], B [B, K, N]
+ *   AITAMD_LAYOUT_CCR: A [B, K, M], B [B, N, K]     AITAMD_LAYOUT_CRR: A [B, K, M], B [B, K, N]
+ * lda / ldb are the row pitches of the matrices as stored, the strides are per batch (0 broadcasts).  d1 = 0
+ * stores plainly with ldc / stride_c; d1 > 0 stores [B/d1, M, d1, N] as aitamd_bmm_rcr_permute does (ldc and
+ * stride_c are ignored).  A transposed operand needs a row pitch that is a multiple of 8 elements.
+ * Replaces the DeviceBatchedGemmXdl / DeviceGemm instances behind bmm_rrr, bmm_ccr, bmm_crr, gemm_rrr and
+ * bmm_rrr_permute (python/aitemplate/backend/rocm/gemm/bmm_rrr.py, bmm_ccr.py, bmm_crr.py, gemm_rrr.py,
+ * bmm_rrr_permute.py; layouts in backend/rocm/gemm/layout.py). */
+enum { AITAMD_LAYOUT_RCR = 0, AITAMD_LAYOUT_RRR = 1, AITAMD_LAYOUT_CCR = 2, AITAMD_LAYOUT_CRR = 3 };
+AITAMD_API int aitamd_bmm(int layout, int dtype, int algo, const void* a, const void* b, void* c,
+                          int64_t batch, int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldc,
+                          int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t d1, void* stream);
+/* aitamd_gemm_algo_supported / aitamd_gemm_heuristic_algo for a given operand layout (same arguments otherwise) */
+AITAMD_API int aitamd_gemm_algo_supported_layout(int epilogue, int dtype, int layout, int algo,
+                                                 int64_t M, int64_t N, int64_t K,
+                                                 int64_t lda, int64_t ldb, int align_bytes);
+AITAMD_API int aitamd_gemm_heuristic_algo_layout(int epilogue, int dtype, int layout, int64_t batch,
+                                                 int64_t M, int64_t N, int64_t K,
+                                                 int64_t lda, int64_t ldb, int align_bytes);
+
 /* bmm_rcr whose [B, M, N] result, viewed as [B/d1, d1, M, N], is written as [B/d1, M, d1, N] (the reference's
  * "0213" permutation with shape = (d1,)): rows of one (batch, head) pair are d1*N elements apart.
  * Replaces the DeviceBatchedGemmEPermuteXdl instances behind bmm_rcr_permute

@@ -180,6 +180,22 @@ def torch_bmm_rcr(q, k) -> torch.Tensor:
     return torch.matmul(q, k.transpose(-1, -2))
 
 
+def torch_bmm(layout: str, a, b) -> torch.Tensor:
+    """fp32 batched product for the reference's operand layouts, as its tests state them
+    (tests/unittest/ops/test_bmm.py:46-50 rcr, :87-89 crr, :120-122 rrr, :153-155 ccr):
+    first letter c = A is [B, K, M] and enters transposed, second letter c = B is [B, N, K] and enters transposed."""
+    a, b = _f(a), _f(b)
+    if a.dim() == 2:
+        a = a.unsqueeze(0)
+    if b.dim() == 2:
+        b = b.unsqueeze(0)
+    if layout[0] == "c":
+        a = a.transpose(-1, -2)
+    if layout[1] == "c":
+        b = b.transpose(-1, -2)
+    return torch.matmul(a, b)
+
+
 def torch_bmm_rcr_permute(q, k, d1: int) -> torch.Tensor:
     """bmm(Q, K^T).reshape(B // d1, d1, M, N).permute(0, 2, 1, 3), as the reference's op states it
     (python/aitemplate/compiler/ops/gemm_universal/bmm_rcr_permute.py:36-45, tests/unittest/ops/test_bmm_permute.py)."""

@@ -365,3 +365,60 @@ def test_bmm_rcr_permute(B, M, N, K, d1, copy_op):      # tests/unittest/ops/tes
     want = oracle.torch_bmm_rcr_permute(q, k, d1).half().float()
     torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
     module.close()
+
+
+# ---- operand layouts other than rcr --------------------------------------------------------------
+@pytest.mark.parametrize("op_name,layout,B,M,N,K", [
+    ("bmm_crr", "crr", 1024, 256, 512, 128),   # test_bmm.py:105-106
+    ("bmm_rrr", "rrr", 87, 23, 512, 256),      # test_bmm.py:138-139
+    ("bmm_ccr", "ccr", 77, 256, 64, 128),      # test_bmm.py:166-167
+    ("bmm_rrr", "rrr", 16, 384, 64, 384),      # probabilities x values of a BERT-base head
+])
+def test_bmm_layouts(op_name, layout, B, M, N, K):
+    print(f"case compile_model {op_name} B={B} M={M} N={N} K={K}", flush=True)
+    a_shape = [B, K, M] if layout[0] == "c" else [B, M, K]
+    b_shape = [B, N, K] if layout[1] == "c" else [B, K, N]
+    X = Tensor(shape=a_shape, dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=b_shape, dtype="float16", name="input_1", is_input=True)
+    Y = _mark_output(getattr(ops, op_name)()(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"{op_name}_{next(_counter)}")
+    a, b = _rand(tuple(a_shape), 1), _rand(tuple(b_shape), 2, K ** -0.5)
+    y = torch.empty(B, M, N, dtype=torch.float16, device="cuda")
+    out = module.run_with_tensors({"input_0": a.cuda(), "input_1": b.cuda()}, [y])
+    assert tuple(out["output_0"].shape) == (B, M, N)
+    torch.testing.assert_close(y.cpu().float(), oracle.torch_bmm(layout, a, b).half().float(), atol=1e-2, rtol=1e-2)
+    module.close()
+
+
+@pytest.mark.parametrize("Ms,K,N", [([256], 128, 32), ([1, 99, 1024, 2048], 256, 16)])
+def test_gemm_rrr(Ms, K, N):                    # tests/unittest/ops/test_gemm.py:226-231
+    print(f"case compile_model gemm_rrr Ms={Ms} K={K} N={N}", flush=True)
+    m_dim = shape_utils.gen_int_var_min_max(Ms, name="m")
+    X = Tensor(shape=[m_dim, IntImm(K)], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[IntImm(K), IntImm(N)], dtype="float16", name="input_1", is_input=True)
+    Y = _mark_output(ops.gemm_rrr()(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"gemm_rrr_{next(_counter)}")
+    for M in Ms:
+        a, b = _rand((M, K), 1), _rand((K, N), 2, K ** -0.5)
+        y = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        module.run_with_tensors({"input_0": a.cuda(), "input_1": b.cuda()}, [y])
+        want = oracle.torch_bmm("rrr", a, b)[0].half().float()
+        torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()
+
+
+def test_bmm_rrr_permute_op():                  # tests/unittest/ops/test_bmm_permute.py:36-71
+    B, M, N, K, d1 = 24, 80, 88, 64, 12
+    print("case compile_model bmm_rrr_permute", flush=True)
+    X = Tensor(shape=[B, M, K], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[B, K, N], dtype="float16", name="input_1", is_input=True)
+    OP = ops.bmm_rrr_permute(shape=(d1,))
+    OP = ops.bmm_rrr_permute(**OP._get_op_attributes())
+    Y = _mark_output(OP(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"bmm_rrr_permute_{next(_counter)}")
+    a, b = _rand((B, M, K), 1), _rand((B, K, N), 2, K ** -0.5)
+    y = torch.empty(B // d1, M, d1, N, dtype=torch.float16, device="cuda")
+    module.run_with_tensors({"input_0": a.cuda(), "input_1": b.cuda()}, [y])
+    want = oracle.torch_bmm("rrr", a, b).reshape(B // d1, d1, M, N).permute(0, 2, 1, 3).half().float()
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()

@@ -481,6 +481,32 @@ def test_bmm_rcr_permute_op_attrs():
         assert registry.exists(f"rocm.bmm_rcr_permute.{hook}")
 
 
+def test_bmm_layout_ops_shapes_keys_and_hooks():
+    """Operand shapes of bmm_xxx.py:204-260 and the reference's exec keys (B, M, N, K order)."""
+    B, M, N, K = 6, 40, 24, 16
+    cases = {"bmm_rrr": ([B, M, K], [B, K, N]), "bmm_ccr": ([B, K, M], [B, N, K]), "bmm_crr": ([B, K, M], [B, K, N])}
+    detect_target()
+    for name, (a_shape, b_shape) in cases.items():
+        op = getattr(ops, name)()
+        y = op(Tensor(a_shape, name="a", is_input=True), Tensor(b_shape, name="b", is_input=True))
+        assert [d.value() for d in y.shape()] == [B, M, N] and op._attrs["op"] == name
+        op._extract_exec_path(DynamicProfileStrategy.MAX)
+        assert list(op._attrs["exec_path"]) == [f"B == {B} && M == {M} && N == {N} && K == {K}"]
+        for hook in ("config", "filter", "gen_profiler", "select_algo", "gen_function", "func_decl", "func_call"):
+            assert registry.exists(f"rocm.{name}.{hook}")
+    with pytest.raises(RuntimeError, match="same K"):
+        ops.bmm_rrr()(Tensor([2, 8, 16], name="a", is_input=True), Tensor([2, 8, 16], name="b", is_input=True))
+    g = ops.gemm_rrr()
+    y = g(Tensor([5, 7, 16], name="a3", is_input=True), Tensor([16, 24], name="b2", is_input=True))
+    assert [d.value() for d in y.shape()] == [5, 7, 24]
+    g._extract_exec_path(DynamicProfileStrategy.MAX)
+    assert list(g._attrs["exec_path"]) == ["M == 35 && N == 24 && K == 16"]
+    p = ops.bmm_rrr_permute(shape=(3,))
+    yp = p(Tensor([B, M, K], name="pa", is_input=True), Tensor([B, K, N], name="pb", is_input=True))
+    assert [d.value() for d in yp.shape()] == [2, M, 3, N] and p._attrs["op"] == "bmm_rrr_permute"
+    assert ops.bmm_rrr_permute(**p._get_op_attributes())._attrs["shape"] == (3,)
+
+
 def test_split_is_a_view_with_byte_offsets():
     x = Tensor([3, 2, 4, 8, 16], name="x", is_input=True)
     q, k, v = ops.split()(x, 1, dim=0)

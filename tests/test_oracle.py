@@ -287,3 +287,23 @@ def test_bmm_rcr_permute_places_each_batch_as_a_head():
     for b in range(B):
         want = q[b].float() @ k[b].float().T
         assert torch.allclose(out[b // d1, :, b % d1, :], want, atol=1e-5)
+
+
+@pytest.mark.parametrize("layout", ["rcr", "rrr", "ccr", "crr"])
+def test_bmm_layouts_brute_force(layout):
+    """C[b, m, n] = sum_k A(b, m, k) B(b, k, n) with the operands indexed as each layout stores them."""
+    B, M, N, K = 2, 3, 4, 5
+    a = _rand((B, K, M) if layout[0] == "c" else (B, M, K), seed=1)
+    b = _rand((B, N, K) if layout[1] == "c" else (B, K, N), seed=2)
+    got = oracle.torch_bmm(layout, a, b)
+    for bi in range(B):
+        for m in range(M):
+            for n in range(N):
+                acc = 0.0
+                for k in range(K):
+                    av = a[bi, k, m] if layout[0] == "c" else a[bi, m, k]
+                    bv = b[bi, n, k] if layout[1] == "c" else b[bi, k, n]
+                    acc += float(av) * float(bv)
+                assert abs(got[bi, m, n].item() - acc) < 1e-4
+    if layout == "rcr":
+        assert torch.equal(got, oracle.torch_bmm_rcr(a, b))
