@@ -43,7 +43,8 @@ EPILOGUE_OF_OP = {
     "gemm_rcr_bias_mul_tanh": 16,
 }
 NUM_RESIDUALS_OF_EPILOGUE = {0: 0, 1: 0, 2: 0, 3: 0, 4: 1, 5: 2, 6: 1, 7: 2, 8: 0, 9: 0,
-                             10: 0, 11: 0, 12: 1, 13: 2, 14: 1, 15: 1, 16: 1}
+                             10: 0, 11: 0, 12: 1, 13: 2, 14: 1, 15: 1, 16: 1, 17: 1}
+EPI_ADD = 17  # residual without bias: the bmm_*_add ops
 DTYPE_ID = {"float16": 0, "bfloat16": 1}
 
 # Ops that store through a 5-D output permutation: name -> (epilogue id, layout id of aitamd_gemm_rcr_permute).
@@ -52,13 +53,16 @@ DTYPE_ID = {"float16": 0, "bfloat16": 1}
 PERMUTE_M2N3, PERMUTE_M3N2 = 1, 2
 LAYOUT_ID = {"rcr": 0, "rrr": 1, "ccr": 2, "crr": 3}
 # plain-epilogue ops launched through aitamd_bmm / aitamd_bmm_rcr_permute
-LAYOUT_OPS = ("bmm_rcr_permute", "bmm_rrr", "bmm_rrr_permute", "bmm_ccr", "bmm_crr", "gemm_rrr")
+LAYOUT_OPS = ("bmm_rcr_permute", "bmm_rrr", "bmm_rrr_permute", "bmm_ccr", "bmm_crr", "gemm_rrr",
+              "bmm_rrr_add", "bmm_ccr_add", "bmm_crr_add")
 PERMUTE_OPS = {
     "gemm_rcr_permute_m2n3": (0, PERMUTE_M2N3),
     "gemm_rcr_bias_permute_m2n3": (1, PERMUTE_M2N3),
     "gemm_rcr_bias_permute_m3n2": (1, PERMUTE_M3N2),
     "gemm_rcr_bias_permute": (1, PERMUTE_M3N2),
+    "gemm_rrr_bias_permute": (1, PERMUTE_M3N2),  # B is [K, N]: operand layout rrr
 }
+PERMUTE_OPERANDS = {"gemm_rrr_bias_permute": "rrr"}  # every other permuting op is rcr
 
 # Every symbol include/aitemplate_amd_kernels.h declares.
 EXPORTED_SYMBOLS = [
@@ -73,6 +77,8 @@ EXPORTED_SYMBOLS = [
     "aitamd_gemm_rcr_permute",
     "aitamd_bmm_rcr_permute",
     "aitamd_bmm",
+    "aitamd_bmm_add",
+    "aitamd_gemm_permute",
     "aitamd_gemm_algo_supported_layout",
     "aitamd_gemm_heuristic_algo_layout",
     "aitamd_bmm_rcr",
@@ -122,6 +128,10 @@ def load() -> ctypes.CDLL:
         lib.aitamd_bmm_rcr_permute.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, vp]
         lib.aitamd_bmm.restype = i32
         lib.aitamd_bmm.argtypes = [i32, i32, i32, vp, vp, vp] + [i64] * 11 + [vp]
+        lib.aitamd_bmm_add.restype = i32
+        lib.aitamd_bmm_add.argtypes = [i32, i32, i32, vp, vp, vp, vp] + [i64] * 12 + [vp]
+        lib.aitamd_gemm_permute.restype = i32
+        lib.aitamd_gemm_permute.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, i64, i64, i64, vp]
         lib.aitamd_gemm_algo_supported_layout.restype = i32
         lib.aitamd_gemm_algo_supported_layout.argtypes = [i32, i32, i32, i32, i64, i64, i64, i64, i64, i32]
         lib.aitamd_gemm_heuristic_algo_layout.restype = i32

@@ -15,7 +15,16 @@ from ...target import Target
 # op -> operand layout ("r": K-contiguous A / [K, N] B; "c": [K, M] A / K-contiguous B), as in
 # python/aitemplate/backend/rocm/gemm/layout.py
 LAYOUT_OF_OP = {"bmm_rcr": "rcr", "bmm_rcr_permute": "rcr", "bmm_rrr": "rrr", "bmm_rrr_permute": "rrr",
-                "bmm_ccr": "ccr", "bmm_crr": "crr", "gemm_rrr": "rrr"}
+                "bmm_ccr": "ccr", "bmm_crr": "crr", "gemm_rrr": "rrr",
+                "bmm_rrr_add": "rrr", "bmm_ccr_add": "ccr", "bmm_crr_add": "crr"}
+
+
+def _is_add(func_attrs) -> bool:
+    return func_attrs["op"].endswith("_add")
+
+
+def _epi(func_attrs) -> int:
+    return _kernels.EPI_ADD if _is_add(func_attrs) else 0
 
 
 def _layout(func_attrs):
@@ -45,7 +54,7 @@ def _filter(instance_name, func_attrs, ab_alignment) -> bool:
     for key in func_attrs["exec_path"]:
         m, n, k = gemm_inverse_key_func(key)[-3:]
         lda, ldb = _pitches(func_attrs, m, n, k)
-        if not lib.aitamd_gemm_algo_supported_layout(0, dtype, lay, algo, m, n, k, lda, ldb,
+        if not lib.aitamd_gemm_algo_supported_layout(_epi(func_attrs), dtype, lay, algo, m, n, k, lda, ldb,
                                                      max(2, min(16, ab_alignment * 2))):
             return False
     return True
@@ -59,15 +68,16 @@ def _select_algo(func_attrs, exec_key) -> str:
     m, n, k = dims[-3:]
     batch = dims[0] if len(dims) == 4 else 1
     lda, ldb = _pitches(func_attrs, m, n, k)
-    algo = lib.aitamd_gemm_heuristic_algo_layout(0, dtype, lay, batch, m, n, k, lda, ldb, 16)
-    all_names = _kernels.gemm_algo_names(0, dtype)
+    algo = lib.aitamd_gemm_heuristic_algo_layout(_epi(func_attrs), dtype, lay, batch, m, n, k, lda, ldb, 16)
+    all_names = _kernels.gemm_algo_names(_epi(func_attrs), dtype)
     if algo >= 0 and all_names[algo] in func_attrs["op_instance"]:
         return all_names[algo]
     return Target.current().select_minimal_algo(list(func_attrs["op_instance"].keys()))
 
 
-def _signature(func_name: str, ranks, permute: bool = False) -> str:
-    ptrs = ["void* in_ptr", "void* weight_ptr", "void* out_ptr"]
+def _signature(func_name: str, ranks, permute: bool = False, add: bool = False) -> str:
+    # the residual of the *_add ops travels as `bias_ptr`, as in the reference (backend/rocm/gemm/common.py:135-137)
+    ptrs = ["void* in_ptr", "void* weight_ptr", "void* out_ptr"] + (["void* bias_ptr"] if add else [])
     dims = [f"int64_t* {n}" for prefix, r in zip("abc", ranks) for n in common.dim_param_names(prefix, r)]
     pdims = ["const int p_dim0"] if permute else []
     return f"void {func_name}({', '.join(ptrs + dims + pdims + ['hipStream_t stream'])})"
@@ -101,11 +111,23 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
     if permute and (off_c or ldc is not None):
         raise NotImplementedError(f"{func_attrs['op']} writes a contiguous permuted buffer; its output cannot be a view")
     plain_rcr = layout == "rcr" and not permute
+    add = _is_add(func_attrs)
+    epi = _epi(func_attrs)
+    ldd = "N"
+    if add:
+        off_d, pitch_d = common.accessor_offset_and_pitch(func_attrs["input_accessors"][2], "d0")
+        if off_d:
+            raise NotImplementedError(f"{func_attrs['op']}: the residual cannot be an offset view")
+        if pitch_d is not None:
+            ldd = str(pitch_d)
     launches = []
     for key, item in func_attrs["exec_path"].items():
         if not item.algo:
             raise RuntimeError(f"{func_name}: workload {key} has no kernel instance; run profiling first")
-        if plain_rcr:
+        if add:
+            call = (f"aitamd_bmm_add({_kernels.LAYOUT_ID[layout]}, {dtype}, algo, a, b, bias_ptr, c, B, M, N, K, lda, ldb, "
+                    f"ldc, {ldd}, stride_a, stride_b, stride_c, M * {ldd}, stream)")
+        elif plain_rcr:
             call = (f"aitamd_bmm_rcr({dtype}, algo, a, b, c, B, M, N, K, lda, ldb, ldc, stride_a, stride_b, stride_c, "
                     "stream)")
         elif layout == "rcr":
@@ -115,12 +137,12 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
             call = (f"aitamd_bmm({_kernels.LAYOUT_ID[layout]}, {dtype}, algo, a, b, c, B, M, N, K, lda, ldb, ldc, "
                     f"stride_a, stride_b, stride_c, {'p_dim0' if permute else '0'}, stream)")
         program = (
-            f'static const int algo = resolve_instance(0, {dtype}, "{item.algo}");\n'
+            f'static const int algo = resolve_instance({epi}, {dtype}, "{item.algo}");\n'
             f'    check_rc({call}, "{func_name}");'
         )
         launches.append(exec_cond_template.format(indent="  ", cond=item.exec_cond, program=program))
     return f"""{common.HEADER}
-{_signature(func_name, (ra, rb, rc), permute)} {{
+{_signature(func_name, (ra, rb, rc), permute, add)} {{
 {shape_code}
   const uint16_t* a = static_cast<const uint16_t*>(in_ptr) + {off_a};
   const uint16_t* b = static_cast<const uint16_t*>(weight_ptr) + {off_b};
@@ -141,7 +163,7 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
 
 
 def func_decl(func_attrs) -> str:
-    return _signature(func_attrs["name"], _ranks(func_attrs), _is_permute(func_attrs)) + ";"
+    return _signature(func_attrs["name"], _ranks(func_attrs), _is_permute(func_attrs), _is_add(func_attrs)) + ";"
 
 
 def func_call(func_attrs, indent="  ") -> str:
@@ -152,7 +174,8 @@ def func_call(func_attrs, indent="  ") -> str:
                 func_attrs["output_accessors"][0]):
         dims += ["&" + d._attrs["name"] for d in acc.original_shapes]
     pdims = [str(int(func_attrs["shape"][0]))] if _is_permute(func_attrs) else []
-    args = [a._attrs["name"], b._attrs["name"], c._attrs["name"]] + dims + pdims + ["stream"]
+    extra = [func_attrs["inputs"][2]._attrs["name"]] if _is_add(func_attrs) else []
+    args = [a._attrs["name"], b._attrs["name"], c._attrs["name"]] + extra + dims + pdims + ["stream"]
     return f"{indent}{func_attrs['name']}({', '.join(args)});"
 
 

@@ -37,7 +37,7 @@ def epilogue_id(op_name: str) -> int:
     if op_name in _kernels.PERMUTE_OPS:
         return _kernels.PERMUTE_OPS[op_name][0]
     if op_name in _kernels.LAYOUT_OPS:
-        return 0
+        return _kernels.EPI_ADD if op_name.endswith("_add") else 0
     return _kernels.EPILOGUE_OF_OP[op_name]
 
 

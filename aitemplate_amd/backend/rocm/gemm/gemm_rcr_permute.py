@@ -1,5 +1,5 @@
 """Registry hooks of the permuting GEMMs: gemm_rcr_permute_m2n3, gemm_rcr_bias_permute,
-gemm_rcr_bias_permute_m2n3 and gemm_rcr_bias_permute_m3n2.
+gemm_rcr_bias_permute_m2n3, gemm_rcr_bias_permute_m3n2 and gemm_rrr_bias_permute (B stored [K, N]).
 
 Replaces python/aitemplate/backend/rocm/gemm/gemm_rcr_permute_m2n3.py, gemm_rcr_bias_permute.py,
 gemm_rcr_bias_permute_m2n3.py:30-160 and gemm_rcr_bias_permute_m3n2.py with their stride tables in
@@ -8,10 +8,16 @@ then `const int p_dim0, p_dim1, p_dim2` (the op's shape attribute) before the st
 from typing import Any, Dict
 
 from .... import _kernels
+from ....compiler.ops.gemm_universal.gemm_common import gemm_inverse_key_func
 from ... import registry
+from ...target import Target
 from . import common
 
 PERMUTE_OPS = list(_kernels.PERMUTE_OPS)
+
+
+def _operands(op: str) -> int:
+    return _kernels.LAYOUT_ID[_kernels.PERMUTE_OPERANDS.get(op, "rcr")]
 
 
 def _ranks(func_attrs):
@@ -46,8 +52,8 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
             raise RuntimeError(f"{func_name}: workload {key} has no kernel instance; run profiling first")
         program = (
             f'static const int algo = resolve_instance({epi}, {dtype}, "{item.algo}");\n'
-            f"    check_rc(aitamd_gemm_rcr_permute({epi}, {dtype}, algo, a, b, {bias_arg}, out_ptr, M, N, K, lda, ldb, "
-            f'{layout}, p_dim0, p_dim1, p_dim2, stream), "{func_name}");'
+            f"    check_rc(aitamd_gemm_permute({_operands(op)}, {epi}, {dtype}, algo, a, b, {bias_arg}, out_ptr, M, N, K, "
+            f'lda, ldb, {layout}, p_dim0, p_dim1, p_dim2, stream), "{func_name}");'
         )
         launches.append(exec_cond_template.format(indent="  ", cond=item.exec_cond, program=program))
     return f"""{common.HEADER}
@@ -56,7 +62,7 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
   const uint16_t* a = static_cast<const uint16_t*>(in_ptr) + {off_a};
   const uint16_t* b = static_cast<const uint16_t*>(weight_ptr) + {off_b};
   const int64_t lda = {lda if lda is not None else "K"};
-  const int64_t ldb = {ldb if ldb is not None else "K"};
+  const int64_t ldb = {ldb if ldb is not None else ("N" if _operands(op) & 1 else "K")};
   if (M == 0 || N == 0) return;  // empty output
 {"".join(launches)}
   throw std::runtime_error(
@@ -81,11 +87,42 @@ def _config(func_attrs, dtype="float16"):
     common.gemm_config(func_attrs, dtype, "gemm_permute")
 
 
+def _filter(instance_name, func_attrs, ab_alignment) -> bool:
+    operands = _operands(func_attrs["op"])
+    if operands == 0:
+        return common.gemm_filter(instance_name, func_attrs, ab_alignment)
+    lib = _kernels.load()
+    dtype = common.DTYPE_ID[func_attrs["inputs"][0]._attrs["dtype"]]
+    epi = _kernels.PERMUTE_OPS[func_attrs["op"]][0]
+    algo = func_attrs["op_instance"][instance_name]
+    for key in func_attrs["exec_path"]:
+        m, n, k = gemm_inverse_key_func(key)[-3:]
+        if not lib.aitamd_gemm_algo_supported_layout(epi, dtype, operands, algo, m, n, k, k, n,
+                                                     max(2, min(16, ab_alignment * 2))):
+            return False
+    return True
+
+
+def _select_algo(func_attrs, exec_key) -> str:
+    operands = _operands(func_attrs["op"])
+    if operands == 0:
+        return common.gemm_select_algo(func_attrs, exec_key)
+    lib = _kernels.load()
+    dtype = common.DTYPE_ID[func_attrs["inputs"][0]._attrs["dtype"]]
+    epi = _kernels.PERMUTE_OPS[func_attrs["op"]][0]
+    m, n, k = gemm_inverse_key_func(exec_key)[-3:]
+    algo = lib.aitamd_gemm_heuristic_algo_layout(epi, dtype, operands, 1, m, n, k, k, n, 16)
+    all_names = _kernels.gemm_algo_names(epi, dtype)
+    if algo >= 0 and all_names[algo] in func_attrs["op_instance"]:
+        return all_names[algo]
+    return Target.current().select_minimal_algo(list(func_attrs["op_instance"].keys()))
+
+
 for _op in PERMUTE_OPS:
     registry.reg(f"rocm.{_op}.config", _config)
-    registry.reg(f"rocm.{_op}.filter", common.gemm_filter)
+    registry.reg(f"rocm.{_op}.filter", _filter)
     registry.reg(f"rocm.{_op}.gen_profiler", common.gemm_gen_profiler)
-    registry.reg(f"rocm.{_op}.select_algo", common.gemm_select_algo)
+    registry.reg(f"rocm.{_op}.select_algo", _select_algo)
     registry.reg(f"rocm.{_op}.gen_function", gen_function)
     registry.reg(f"rocm.{_op}.func_decl", func_decl)
     registry.reg(f"rocm.{_op}.func_call", func_call)

@@ -189,3 +189,42 @@ class bmm_rrr_permute(bmm_rrr):
 
     __call__ = bmm_rcr_permute.__call__
     _get_op_attributes = bmm_rcr_permute._get_op_attributes
+
+
+def _add_class(base, name: str):
+    """base(A, B) + D with D of the result's shape [B, M, N]
+    (python/aitemplate/compiler/ops/gemm_universal/bmm_xxx_add.py:21-64)."""
+
+    class _bmm_add(base):
+        __doc__ = f"C[b] = {base.__name__}(A, B)[b] + D[b]"
+
+        def __init__(self):
+            super().__init__()
+            self._attrs["op"] = name
+            self._attrs["num_sources"] = 1
+
+        @classmethod
+        def is_valid_inputs(cls, a: Tensor, b: Tensor, d: Tensor):
+            out = base()._infer_shapes(a, b)
+            if list(d.shape()) != list(out):
+                return False, f"Additional elementwise shape {d.shape()} doesn't match bmm's shape {out}"
+            return True, ""
+
+        def __call__(self, a: Tensor, b: Tensor, d: Tensor) -> Tensor:
+            a, b = self._align_ab(a, b)
+            ok, msg = self.is_valid_inputs(a, b, d)
+            if not ok:
+                raise RuntimeError(msg)
+            self._attrs["inputs"] = [a, b, d]
+            self._attrs["input_accessors"] = [TensorAccessor(t) for t in self._attrs["inputs"]]
+            self._set_depth()
+            self._sanity_check(a, b)
+            return self._finish_call([a, b, d], self._infer_shapes(a, b))
+
+    _bmm_add.__name__ = _bmm_add.__qualname__ = name
+    return _bmm_add
+
+
+bmm_rrr_add = _add_class(bmm_rrr, "bmm_rrr_add")
+bmm_ccr_add = _add_class(bmm_ccr, "bmm_ccr_add")
+bmm_crr_add = _add_class(bmm_crr, "bmm_crr_add")

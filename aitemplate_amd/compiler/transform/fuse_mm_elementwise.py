@@ -1,8 +1,7 @@
 """Fold chains of element-wise ops behind a GEMM into the fused GEMM ops.
 
 Counterpart of python/aitemplate/compiler/transform/fuse_mm_elementwise.py:31-215 with the pattern table of
-fuse_mm_elementwise_patterns.py:46-200 (the gemm_rcr rows; the bmm_*_add ops and the bmm alpha fold have
-no kernels in this backend).  Matching is by chain: starting at a gemm_rcr / gemm_rcr_bias output, follow
+fuse_mm_elementwise_patterns.py:46-200 (the bmm alpha fold is left out: the kernels take no alpha).  Matching is by chain: starting at a gemm_rcr / gemm_rcr_bias output, follow
 tensors that have exactly one consumer, an element-wise op, and are not graph outputs; the longest prefix of
 the chain that is a row of the table is replaced.  Binary steps (ADD, MUL) take the other operand as the
 fused op's residual, and the replacement's own `is_valid_inputs` decides whether it fits (the residual must
@@ -21,6 +20,9 @@ _BINARY = {_F.ADD, _F.MUL}
 
 # (first op, element-wise chain) -> fused op, as in the reference's table
 PATTERNS = {
+    ("bmm_ccr", (_F.ADD,)): "bmm_ccr_add",
+    ("bmm_crr", (_F.ADD,)): "bmm_crr_add",
+    ("bmm_rrr", (_F.ADD,)): "bmm_rrr_add",
     ("gemm_rcr", (_F.ADD,)): "gemm_rcr_bias",
     ("gemm_rcr_bias", (_F.RELU,)): "gemm_rcr_bias_relu",
     ("gemm_rcr_bias", (_F.SIGMOID, _F.MUL, _F.TANH)): "gemm_rcr_bias_sigmoid_mul_tanh",
@@ -38,6 +40,7 @@ PATTERNS = {
     ("gemm_rcr_bias", (_F.MUL,)): "gemm_rcr_bias_mul",
 }
 _MAX_CHAIN = max(len(k[1]) for k in PATTERNS)
+_START_OPS = {k[0] for k in PATTERNS}
 
 
 def _only_consumer(t: Tensor) -> Optional[Operator]:
@@ -144,7 +147,7 @@ def fuse_mm_elementwise(sorted_graph: List[Tensor], output_tensors: List[Tensor]
         changed = False
         for t in sorted_graph:
             for op in list(t.src_ops()):
-                if op._attrs["op"] in ("gemm_rcr", "gemm_rcr_bias") and op._attrs["outputs"][0] is t:
+                if op._attrs["op"] in _START_OPS and op._attrs["outputs"][0] is t:
                     if _fuse_chain(op, output_tensors) or _fuse_swish(op, output_tensors):
                         changed = True
                         break

@@ -34,7 +34,8 @@ enum EpilogueId : int {
   kEpiBiasSigmoidMul = 14,  // gemm_rcr_bias_sigmoid_mul
   kEpiBiasSigmoidMulTanh = 15,  // gemm_rcr_bias_sigmoid_mul_tanh
   kEpiBiasMulTanh = 16,     // gemm_rcr_bias_mul_tanh
-  kNumEpilogues = 17,
+  kEpiAdd = 17,             // bmm_rrr_add, bmm_ccr_add, bmm_crr_add: residual without bias
+  kNumEpilogues = 18,
 };
 
 AITAMD_DEVICE float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
@@ -96,6 +97,7 @@ AITAMD_DEF_EPI(kEpiBiasMulAdd, true, 2, (acc + b) * d0 + d1)
 AITAMD_DEF_EPI(kEpiBiasSigmoidMul, true, 1, sigmoid_f(acc + b) * d0)
 AITAMD_DEF_EPI(kEpiBiasSigmoidMulTanh, true, 1, tanh_f(sigmoid_f(acc + b) * d0))
 AITAMD_DEF_EPI(kEpiBiasMulTanh, true, 1, tanh_f((acc + b) * d0))
+AITAMD_DEF_EPI(kEpiAdd, false, 1, acc + d0)
 
 #undef AITAMD_DEF_EPI
 

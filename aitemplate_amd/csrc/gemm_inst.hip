@@ -34,9 +34,11 @@ using Epi = Epilogue<AITAMD_EPI>;
 // Kernels with the permuted store exist for the two epilogues the permuting ops use.
 constexpr bool kHasPermutedStore = AITAMD_EPI == kEpiNone || AITAMD_EPI == kEpiBias;
 
-// Kernels for operands that are not K-contiguous (layouts rrr, ccr, crr) exist for the plain epilogue, on the
-// direct-to-LDS tiles whose edges allow it.
-constexpr bool kHasLayouts = AITAMD_EPI == kEpiNone;
+// Kernels for operands that are not K-contiguous exist on the direct-to-LDS tiles whose edges allow it, for the
+// epilogues the reference's ops in those layouts use: plain and residual-add in all of rrr, ccr, crr; bias for
+// rrr with the permuted store (gemm_rrr_bias_permute).  kLayoutBits: bit L set when layout L is compiled.
+constexpr int kLayoutBits = (AITAMD_EPI == kEpiNone || AITAMD_EPI == kEpiAdd) ? 0xf : (AITAMD_EPI == kEpiBias ? 0x3 : 0x1);
+constexpr bool kLayoutsArePermuted = AITAMD_EPI == kEpiBias;  // the bias kernels of the other layouts store permuted
 
 template <class Tile, bool PERM, int LAYOUT>
 struct KernelOf {
@@ -60,7 +62,7 @@ struct LayoutMask {
 template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
 struct LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>> {
   static constexpr int value =
-      (kHasLayouts && GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kTransposable) ? 0xf : 1;
+      GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kTransposable ? kLayoutBits : 1;
 };
 template <class Tile>
 struct IsPersistent {
@@ -124,13 +126,16 @@ hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
 template <class Tile>
 hipError_t launch_tile(const GemmParams& p, hipStream_t stream) {
   if (p.layout != 0) {
-    if constexpr (LayoutMask<Tile>::value == 0xf) {
-      if (p.perm_on) return hipErrorInvalidValue;
-      switch (p.layout) {
-        case 1: return launch_kernel<Tile, false, 1>(p, stream);
-        case 2: return launch_kernel<Tile, false, 2>(p, stream);
-        case 3: return launch_kernel<Tile, false, 3>(p, stream);
-      }
+    constexpr int mask = LayoutMask<Tile>::value;
+    if ((p.perm_on != 0) != kLayoutsArePermuted) return hipErrorInvalidValue;
+    if constexpr ((mask & 2) != 0) {
+      if (p.layout == 1) return launch_kernel<Tile, kLayoutsArePermuted, 1>(p, stream);
+    }
+    if constexpr ((mask & 4) != 0) {
+      if (p.layout == 2) return launch_kernel<Tile, kLayoutsArePermuted, 2>(p, stream);
+    }
+    if constexpr ((mask & 8) != 0) {
+      if (p.layout == 3) return launch_kernel<Tile, kLayoutsArePermuted, 3>(p, stream);
     }
     return hipErrorInvalidValue;
   }

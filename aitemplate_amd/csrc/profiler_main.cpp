@@ -109,6 +109,7 @@ int epilogue_of(const std::string& op) {
                                 "gemm_rcr_bias_sigmoid_mul_tanh", "gemm_rcr_bias_mul_tanh"};
   if (op == "gemm_rcr_bias_fast_gelu") return AITAMD_EPI_BIAS_GELU;
   if (op == "bmm_rcr") return AITAMD_EPI_NONE;
+  if (op == "bmm_add") return AITAMD_EPI_ADD;
   for (int i = 0; i < AITAMD_NUM_EPILOGUES; ++i)
     if (op == names[i]) return i;
   return -1;
@@ -122,6 +123,7 @@ int num_residuals(int epi) {
     case AITAMD_EPI_BIAS_SIGMOID_MUL:
     case AITAMD_EPI_BIAS_SIGMOID_MUL_TANH:
     case AITAMD_EPI_BIAS_MUL_TANH:
+    case AITAMD_EPI_ADD:
       return 1;
     case AITAMD_EPI_BIAS_ADD_ADD:
     case AITAMD_EPI_BIAS_ADD_ADD_RELU:
@@ -152,7 +154,8 @@ bool permute_op(const std::string& op, std::string* base, int* layout) {
   } table[] = {{"gemm_rcr_permute_m2n3", "gemm_rcr", AITAMD_PERMUTE_M2N3},
                {"gemm_rcr_bias_permute_m2n3", "gemm_rcr_bias", AITAMD_PERMUTE_M2N3},
                {"gemm_rcr_bias_permute_m3n2", "gemm_rcr_bias", AITAMD_PERMUTE_M3N2},
-               {"gemm_rcr_bias_permute", "gemm_rcr_bias", AITAMD_PERMUTE_M3N2}};
+               {"gemm_rcr_bias_permute", "gemm_rcr_bias", AITAMD_PERMUTE_M3N2},
+               {"gemm_rrr_bias_permute", "gemm_rcr_bias", AITAMD_PERMUTE_M3N2}};
   for (const auto& t : table)
     if (op == t.op) {
       *base = t.base;
@@ -210,9 +213,17 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
   HIP_OK(hipEventCreate(&e1));
 
   auto launch = [&](int algo, const OperandSet& o) -> int {
-    if (perm.layout && !batched)
+    if (perm.layout && !batched && perm.operands == AITAMD_LAYOUT_RCR)
       return aitamd_gemm_rcr_permute(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.c.p, M, N, K, K, K, perm.layout,
                                      perm.g[0], perm.g[1], perm.g[2], stream);
+    if (batched && epi == AITAMD_EPI_ADD) {
+      const int64_t lda = (perm.operands & 2) ? M : K, ldb = (perm.operands & 1) ? N : K;
+      return aitamd_bmm_add(perm.operands, dtype, algo, o.a.p, o.b.p, o.d0.p, o.c.p, B, M, N, K, lda, ldb, N, N, M * K,
+                            N * K, M * N, M * N, stream);
+    }
+    if (!batched && perm.layout && perm.operands != AITAMD_LAYOUT_RCR)
+      return aitamd_gemm_permute(perm.operands, epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.c.p, M, N, K, K, N,
+                                 perm.layout, perm.g[0], perm.g[1], perm.g[2], stream);
     if (batched && perm.operands != AITAMD_LAYOUT_RCR) {
       const int64_t lda = (perm.operands & 2) ? M : K, ldb = (perm.operands & 1) ? N : K;
       return aitamd_bmm(perm.operands, dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, lda, ldb, N, M * K, N * K, M * N,
@@ -335,6 +346,7 @@ int main(int argc, char** argv) {
     perm.g[0] = d[3];
     perm.g[1] = d[4];
     perm.g[2] = d[5];
+    if (op == "gemm_rrr_bias_permute") perm.operands = AITAMD_LAYOUT_RRR;
     return profile_gemm_like(base, dtype, 1, d[0], d[1], d[2], false, perm);
   }
   if (kind == "bmm") {
@@ -360,7 +372,8 @@ int main(int argc, char** argv) {
       perm.layout = 1;
       perm.g[0] = d[need];
     }
-    if (batched) return profile_gemm_like("bmm_rcr", dtype, d[0], d[1], d[2], d[3], true, perm);
+    const bool add = op.size() > 4 && op.compare(op.size() - 4, 4, "_add") == 0;
+    if (batched) return profile_gemm_like(add ? "bmm_add" : "bmm_rcr", dtype, d[0], d[1], d[2], d[3], true, perm);
     return profile_gemm_like("bmm_rcr", dtype, 1, d[0], d[1], d[2], true, perm);
   }
   if (kind == "attn") {

@@ -103,11 +103,13 @@ def gemm_permute(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch
         raise ValueError(f"unsupported dtype {dtype}")
     for t, n in ((a, "a"), (b, "b"), (bias, "bias"), (out, "out")):
         _check(t, n, dtype)
+    operands = _kernels.LAYOUT_ID[_kernels.PERMUTE_OPERANDS.get(op, "rcr")]
     K = a.shape[-1]
     a2 = a.reshape(-1, K)
-    M, N = a2.shape[0], b.shape[0]
-    if b.dim() != 2 or b.shape[1] != K:
-        raise ValueError(f"b must be [N, K={K}], got {tuple(b.shape)}")
+    b_k, b_n = (0, 1) if operands & 1 else (1, 0)  # gemm_rrr_bias_permute takes B as [K, N]
+    if b.dim() != 2 or b.shape[b_k] != K:
+        raise ValueError(f"b does not match K={K}: got {tuple(b.shape)}")
+    M, N = a2.shape[0], b.shape[b_n]
     if epi != 0 and (bias is None or bias.numel() != N):
         raise ValueError("bias must be 1-D of size N")
     t1, t2, t3 = (int(t) for t in shape)
@@ -123,8 +125,8 @@ def gemm_permute(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch
         out = torch.empty(out_shape, dtype=dtype, device=a.device)
     elif not out.is_contiguous() or out.numel() != M * N:
         raise ValueError("out must be contiguous with M*N elements")
-    rc = lib.aitamd_gemm_rcr_permute(epi, _TORCH_DTYPE_ID[dtype], algo, _p(a2), _p(b), _p(bias), _p(out), M, N, K,
-                                     _row_pitch(a2, "a"), _row_pitch(b, "b"), layout, t1, t2, t3, _stream_ptr())
+    rc = lib.aitamd_gemm_permute(operands, epi, _TORCH_DTYPE_ID[dtype], algo, _p(a2), _p(b), _p(bias), _p(out), M, N, K,
+                                 _row_pitch(a2, "a"), _row_pitch(b, "b"), layout, t1, t2, t3, _stream_ptr())
     _kernels.check(rc, op)
     return out
 
@@ -190,6 +192,32 @@ def bmm(layout: str, a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tenso
     rc = lib.aitamd_bmm(lay, _TORCH_DTYPE_ID[dtype], algo, _p(a3), _p(b3), _p(out), B, M, N, K, a3.shape[2],
                         b3.shape[2], N, sa, sb, M * N, d1, _stream_ptr())
     _kernels.check(rc, f"bmm_{layout}")
+    return out
+
+
+def bmm_add(layout: str, a: torch.Tensor, b: torch.Tensor, d0: torch.Tensor, out: Optional[torch.Tensor] = None,
+            algo: int = -1) -> torch.Tensor:
+    """bmm(layout, a, b) + d0 with d0 of the result's shape [B, M, N]: the bmm_rrr_add / bmm_ccr_add / bmm_crr_add
+    ops (python/aitemplate/compiler/ops/gemm_universal/bmm_xxx_add.py)."""
+    lib = _kernels.load()
+    lay = _kernels.LAYOUT_ID[layout]
+    dtype = a.dtype
+    for t, n in ((a, "a"), (b, "b"), (d0, "d0"), (out, "out")):
+        _check(t, n, dtype)
+    if a.dim() != 3 or b.dim() != 3 or not (a.is_contiguous() and b.is_contiguous() and d0.is_contiguous()):
+        raise ValueError("bmm_add operands must be contiguous 3-D tensors")
+    B = a.shape[0]
+    M, K = (a.shape[2], a.shape[1]) if lay & 2 else (a.shape[1], a.shape[2])
+    N, Kb = (b.shape[2], b.shape[1]) if lay & 1 else (b.shape[1], b.shape[2])
+    if Kb != K or b.shape[0] != B:
+        raise ValueError("A and B do not match")
+    if tuple(d0.shape) != (B, M, N):
+        raise ValueError(f"d0 must be [{B}, {M}, {N}], got {tuple(d0.shape)}")
+    if out is None:
+        out = torch.empty(B, M, N, dtype=dtype, device=a.device)
+    rc = lib.aitamd_bmm_add(lay, _TORCH_DTYPE_ID[dtype], algo, _p(a), _p(b), _p(d0), _p(out), B, M, N, K, a.shape[2],
+                            b.shape[2], N, N, M * K, N * K, M * N, M * N, _stream_ptr())
+    _kernels.check(rc, f"bmm_{layout}_add")
     return out
 
 

@@ -55,7 +55,8 @@ enum {
   AITAMD_EPI_BIAS_SIGMOID_MUL = 14,     /* gemm_rcr_bias_sigmoid_mul  : AddSigmoidMul*/
   AITAMD_EPI_BIAS_SIGMOID_MUL_TANH = 15,/* gemm_rcr_bias_sigmoid_mul_tanh            */
   AITAMD_EPI_BIAS_MUL_TANH = 16,        /* gemm_rcr_bias_mul_tanh     : AddMulTanh   */
-  AITAMD_NUM_EPILOGUES = 17
+  AITAMD_EPI_ADD = 17,                  /* bmm_{rrr,ccr,crr}_add      : acc + D0, no bias */
+  AITAMD_NUM_EPILOGUES = 18
 };
 
 enum { AITAMD_F16 = 0, AITAMD_BF16 = 1 };
@@ -152,6 +153,21 @@ AITAMD_API int aitamd_bmm(int layout, int dtype, int algo, const void* a, const 
                           int64_t batch, int64_t M, int64_t N, int64_t K,
                           int64_t lda, int64_t ldb, int64_t ldc,
                           int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t d1, void* stream);
+/* C[b] = A[b] x B[b] + D0[b] (epilogue AITAMD_EPI_ADD) in any of the four operand layouts; D0 is row-major
+ * [B, M, N] with row pitch ldd and batch stride stride_d (0 broadcasts one [M, N] residual).
+ * Replaces the instances behind bmm_rrr_add, bmm_ccr_add, bmm_crr_add
+ * (python/aitemplate/backend/rocm/gemm/bmm_rrr_add.py, bmm_ccr_add.py, bmm_crr_add.py). */
+AITAMD_API int aitamd_bmm_add(int layout, int dtype, int algo, const void* a, const void* b, const void* d0, void* c,
+                              int64_t batch, int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                              int64_t stride_a, int64_t stride_b, int64_t stride_c, int64_t stride_d, void* stream);
+/* aitamd_gemm_rcr_permute with the operand layout as a parameter: AITAMD_LAYOUT_RCR with epilogues none / bias, or
+ * AITAMD_LAYOUT_RRR (B is [K, N]) with the bias epilogue, which is gemm_rrr_bias_permute
+ * (python/aitemplate/backend/rocm/gemm/gemm_rrr_bias_permute.py:40-110). */
+AITAMD_API int aitamd_gemm_permute(int operands, int epilogue, int dtype, int algo,
+                                   const void* a, const void* b, const void* bias, void* c,
+                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                   int layout, int64_t g1, int64_t g2, int64_t g3, void* stream);
 /* aitamd_gemm_algo_supported / aitamd_gemm_heuristic_algo for a given operand layout (same arguments otherwise) */
 AITAMD_API int aitamd_gemm_algo_supported_layout(int epilogue, int dtype, int layout, int algo,
                                                  int64_t M, int64_t N, int64_t K,

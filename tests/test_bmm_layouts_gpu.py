@@ -96,3 +96,53 @@ def test_unsupported_pitch_is_reported():
         eager.bmm("rrr", a.cuda(), b.cuda())
     assert lib.aitamd_gemm_heuristic_algo_layout(0, 0, 1, 2, 64, 36, 64, 64, 36, 16) == -1
     assert lib.aitamd_bmm(7, 0, -1, None, None, None, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 0, None) != 0
+
+
+# ---- residual add and the rrr bias + permuted store ---------------------------------------------
+@pytest.mark.parametrize("layout,B,M,N,K", [
+    ("rrr", 32, 256, 512, 256), ("ccr", 32, 256, 256, 512), ("crr", 32, 256, 512, 256),   # test_bmm_add.py:286-302
+    ("rcr", 6, 200, 136, 72), ("rrr", 3, 200, 136, 72), ("ccr", 5, 104, 88, 40), ("crr", 2, 520, 64, 33),
+])
+def test_bmm_add(layout, B, M, N, K):
+    print(f"case bmm_{layout}_add B={B} M={M} N={N} K={K}", flush=True)
+    a, b = _operands(layout, B, M, N, K)
+    d = _rand((B, M, N), 7)
+    got = eager.bmm_add(layout, a.cuda(), b.cuda(), d.cuda())
+    torch.cuda.synchronize()
+    want = (oracle.torch_bmm(layout, a, b) + d.float()).half().float()
+    torch.testing.assert_close(got.cpu().float(), want, atol=1e-2, rtol=1e-2)
+
+
+def test_bmm_add_every_instance():
+    lib = _kernels.load()
+    B, M, N, K = 2, 200, 136, 72
+    for layout in ("rcr", "rrr", "ccr", "crr"):
+        lay = _kernels.LAYOUT_ID[layout]
+        a, b = _operands(layout, B, M, N, K, seed=lay)
+        d = _rand((B, M, N), 11)
+        want = (oracle.torch_bmm(layout, a, b) + d.float()).half().float()
+        ad, bd, dd = a.cuda(), b.cuda(), d.cuda()
+        ran = 0
+        for algo, name in enumerate(_kernels.gemm_algo_names(_kernels.EPI_ADD, 0)):
+            if not lib.aitamd_gemm_algo_supported_layout(_kernels.EPI_ADD, 0, lay, algo, M, N, K, a.shape[2], b.shape[2], 16):
+                continue
+            print(f"case bmm_{layout}_add instance={name}", flush=True)
+            got = eager.bmm_add(layout, ad, bd, dd, algo=algo)
+            torch.cuda.synchronize()
+            torch.testing.assert_close(got.cpu().float(), want, atol=1e-2, rtol=1e-2)
+            ran += 1
+        assert ran >= 5
+
+
+@pytest.mark.parametrize("M,N,K,shape", [(4 * 32 * 128, 16 * 256, 128, (32, 128, 16)),   # test_gemm_bias_permute.py:250-280
+                                         (3 * 7 * 8, 5 * 16, 24, (7, 8, 5)), (2 * 3 * 100, 4 * 72, 200, (3, 100, 4))])
+def test_gemm_rrr_bias_permute(M, N, K, shape):
+    print(f"case gemm_rrr_bias_permute M={M} N={N} K={K} shape={shape}", flush=True)
+    x, w, bias = _rand((M, K), 1), _rand((K, N), 2, K ** -0.5), _rand((N,), 3)
+    got = eager.gemm_permute("gemm_rrr_bias_permute", x.cuda(), w.cuda(), bias.cuda(), shape)
+    torch.cuda.synchronize()
+    t1, t2, t3 = shape
+    y = oracle.torch_bmm("rrr", x, w)[0] + bias.float()
+    want = oracle.permute_5d(y, "m3n2", shape).half().float()
+    assert tuple(got.shape) == (t2, M // (t1 * t2), t3, t1, N // t3)
+    torch.testing.assert_close(got.cpu().float(), want, atol=1e-2, rtol=1e-2)

@@ -422,3 +422,43 @@ def test_bmm_rrr_permute_op():                  # tests/unittest/ops/test_bmm_pe
     want = oracle.torch_bmm("rrr", a, b).reshape(B // d1, d1, M, N).permute(0, 2, 1, 3).half().float()
     torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
     module.close()
+
+
+@pytest.mark.parametrize("op_name,layout,B,M,N,K", [("bmm_rrr_add", "rrr", 32, 256, 512, 256),
+                                                     ("bmm_ccr_add", "ccr", 32, 256, 256, 512),
+                                                     ("bmm_crr_add", "crr", 32, 256, 512, 256)])
+def test_bmm_add_ops(op_name, layout, B, M, N, K):      # tests/unittest/ops/test_bmm_add.py:286-302
+    print(f"case compile_model {op_name} B={B} M={M} N={N} K={K}", flush=True)
+    a_shape = [B, K, M] if layout[0] == "c" else [B, M, K]
+    b_shape = [B, N, K] if layout[1] == "c" else [B, K, N]
+    X = Tensor(shape=a_shape, dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=b_shape, dtype="float16", name="input_1", is_input=True)
+    D = Tensor(shape=[B, M, N], dtype="float16", name="input_2", is_input=True)
+    # written unfused: the pass turns bmm + ADD into the fused op
+    Y = _mark_output(getattr(ops, op_name[:-4])()(X, W) + D)
+    name = f"{op_name}_{next(_counter)}"
+    module = compile_model(Y, detect_target(), WORKDIR, name)
+    assert f"{op_name}_" in open(os.path.join(WORKDIR, name, "model-generated.cpp")).read()
+    a, b, d = _rand(tuple(a_shape), 1), _rand(tuple(b_shape), 2, K ** -0.5), _rand((B, M, N), 3)
+    y = torch.empty(B, M, N, dtype=torch.float16, device="cuda")
+    module.run_with_tensors({"input_0": a.cuda(), "input_1": b.cuda(), "input_2": d.cuda()}, [y])
+    want = (oracle.torch_bmm(layout, a, b) + d.float()).half().float()
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()
+
+
+def test_gemm_rrr_bias_permute_op():            # tests/unittest/ops/test_gemm_bias_permute.py:250-280
+    M0, M1, M2, N0, N1, K = 4, 32, 128, 16, 256, 128
+    M, N, shape = M0 * M1 * M2, N0 * N1, (M1, M2, N0)
+    print("case compile_model gemm_rrr_bias_permute", flush=True)
+    X = Tensor(shape=[M, K], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[K, N], dtype="float16", name="input_1", is_input=True)
+    Bv = Tensor(shape=[N], dtype="float16", name="input_2", is_input=True)
+    Y = _mark_output(ops.gemm_rrr_bias_permute(shape)(X, W, Bv))
+    module = compile_model(Y, detect_target(), WORKDIR, f"gemm_rrr_bias_permute_{next(_counter)}")
+    x, w, b = _rand((M, K), 1), _rand((K, N), 2, K ** -0.5), _rand((N,), 3)
+    want = oracle.permute_5d(oracle.torch_bmm("rrr", x, w)[0] + b.float(), "m3n2", shape).half().float()
+    y = torch.empty(tuple(want.shape), dtype=torch.float16, device="cuda")
+    module.run_with_tensors({"input_0": x.cuda(), "input_1": w.cuda(), "input_2": b.cuda()}, [y])
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()

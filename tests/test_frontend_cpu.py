@@ -501,6 +501,22 @@ def test_bmm_layout_ops_shapes_keys_and_hooks():
     assert [d.value() for d in y.shape()] == [5, 7, 24]
     g._extract_exec_path(DynamicProfileStrategy.MAX)
     assert list(g._attrs["exec_path"]) == ["M == 35 && N == 24 && K == 16"]
+    X, W, D = Tensor([B, M, K], name="x", is_input=True), Tensor([B, K, N], name="w", is_input=True), \
+        Tensor([B, M, N], name="d", is_input=True)
+    fused = ops.bmm_rrr()(X, W) + D
+    fused._attrs["is_output"] = True
+    graph, _ = _fuse([fused])
+    assert _op_names(graph) == ["bmm_rrr_add"]
+    with pytest.raises(RuntimeError, match="doesn't match"):
+        ops.bmm_ccr_add()(Tensor([B, K, M], name="xa", is_input=True), Tensor([B, N, K], name="wa", is_input=True),
+                          Tensor([B, M, N + 8], name="da", is_input=True))
+    rp = ops.gemm_rrr_bias_permute((2, 4, 3))
+    yr = rp(Tensor([16, 8], name="rx", is_input=True), Tensor([8, 24], name="rw", is_input=True),
+            Tensor([24], name="rb", is_input=True))
+    assert [d.value() for d in yr.shape()] == [4, 2, 3, 2, 8] and rp._attrs["op"] == "gemm_rrr_bias_permute"
+    for name in ("bmm_rrr_add", "bmm_ccr_add", "bmm_crr_add", "gemm_rrr", "gemm_rrr_bias_permute", "bmm_rrr_permute"):
+        for hook in ("config", "filter", "gen_profiler", "select_algo", "gen_function", "func_decl", "func_call"):
+            assert registry.exists(f"rocm.{name}.{hook}"), f"rocm.{name}.{hook}"
     p = ops.bmm_rrr_permute(shape=(3,))
     yp = p(Tensor([B, M, K], name="pa", is_input=True), Tensor([B, K, N], name="pb", is_input=True))
     assert [d.value() for d in yp.shape()] == [2, M, 3, N] and p._attrs["op"] == "bmm_rrr_permute"
@@ -555,7 +571,7 @@ def test_multihead_attention_block_compiles_to_three_kernels(tmp_path, monkeypat
                                                    "gemm_rcr_bias_add"], entries
     qkv_src = (build / f"{entries[0]}.cpp").read_text()
     assert "const int p_dim0, const int p_dim1, const int p_dim2, hipStream_t stream)" in qkv_src
-    assert "aitamd_gemm_rcr_permute(1, 0, algo, a, b, bias_ptr, out_ptr, M, N, K, lda, ldb, 1, p_dim0, p_dim1, " \
+    assert "aitamd_gemm_permute(0, 1, 0, algo, a, b, bias_ptr, out_ptr, M, N, K, lda, ldb, 1, p_dim0, p_dim1, " \
            "p_dim2, stream)" in qkv_src
     assert f", {S}, 3, {H}, stream);" in model_src
     # K and V are the second and third [B, heads, S, head_dim] pieces of the packed projection
