@@ -228,9 +228,13 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)c.batch * p.sd : nullptr;
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)c.batch * p.sd : nullptr;
     const int n = c.n0 + wn * Tile::WTN + r_c * 8;  // the lane's 8 columns: the same in every pass
-    vec8 bv = {};
+    float bf8[8] = {};  // the lane's 8 bias values, converted once per tile
     if constexpr (Epi::kHasBias) {
-      if (vec_ok && n < p.N) bv = *reinterpret_cast<const vec8*>(bias + n);
+      if (vec_ok && n < p.N) {
+        const vec8 bv = *reinterpret_cast<const vec8*>(bias + n);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) bf8[j] = Tr::to_float(bv[j]);
+      }
     }
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
@@ -263,8 +267,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
             vec8 o;
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-              o[j] = Tr::from_float(Epi::apply(Tr::to_float(raw[j]), Tr::to_float(bv[j]), Tr::to_float(d0v[j]),
-                                               Tr::to_float(d1v[j])));
+              o[j] = Tr::from_float(Epi::apply(Tr::to_float(raw[j]), bf8[j], Tr::to_float(d0v[j]), Tr::to_float(d1v[j])));
             store_out(Cb, c_idx, o, p.nt_store != 0, rc);
           } else {
 #pragma unroll
