@@ -462,3 +462,49 @@ def test_gemm_rrr_bias_permute_op():            # tests/unittest/ops/test_gemm_b
     module.run_with_tensors({"input_0": x.cuda(), "input_1": w.cuda(), "input_2": b.cuda()}, [y])
     torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
     module.close()
+
+
+@pytest.mark.parametrize("op_name,layout,bs,ms,N,K", [
+    ("bmm_rrr", "rrr", [2, 5, 99], [23], 512, 128),          # test_bmm.py:134 dynamic_b
+    ("bmm_rrr", "rrr", [2, 5, 7], [1, 7, 9], 512, 256),      # test_bmm.py:136 dynamic_bm
+    ("bmm_crr", "crr", [3, 977, 1024], [256], 512, 128),     # test_bmm.py:101 dynamic_b
+    ("bmm_ccr", "ccr", [1, 9, 101], [256], 64, 128),         # test_bmm.py:164 dynamic_b
+])
+def test_bmm_layouts_dynamic_dims(op_name, layout, bs, ms, N, K):
+    print(f"case compile_model {op_name} bs={bs} ms={ms} N={N} K={K}", flush=True)
+    b_dim = shape_utils.gen_int_var_min_max(bs, name="batch_size")
+    m_dim = shape_utils.gen_int_var_min_max(ms, name="m")
+    a_shape = [b_dim, IntImm(K), m_dim] if layout[0] == "c" else [b_dim, m_dim, IntImm(K)]
+    b_shape = [b_dim, IntImm(N), IntImm(K)] if layout[1] == "c" else [b_dim, IntImm(K), IntImm(N)]
+    if layout[0] == "c" and len(ms) > 1:
+        pytest.skip("a dynamic pitch of the transposed operand is not a case of the reference either")
+    X = Tensor(shape=a_shape, dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=b_shape, dtype="float16", name="input_1", is_input=True)
+    Y = _mark_output(getattr(ops, op_name)()(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"{op_name}_dyn_{next(_counter)}")
+    for B in bs:
+        for M in ms:
+            a = _rand((B, K, M) if layout[0] == "c" else (B, M, K), B + M)
+            b = _rand((B, N, K) if layout[1] == "c" else (B, K, N), B + M + 1, K ** -0.5)
+            y = torch.empty(B, M, N, dtype=torch.float16, device="cuda")
+            out = module.run_with_tensors({"input_0": a.cuda(), "input_1": b.cuda()}, [y])
+            assert tuple(out["output_0"].shape) == (B, M, N)
+            want = oracle.torch_bmm(layout, a, b).half().float()
+            torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()
+
+
+def test_bmm_crr_dynamic_k():                   # tests/unittest/ops/test_bmm.py:102 (dynamic_k)
+    print("case compile_model bmm_crr dynamic K", flush=True)
+    B, M, N, ks = 5, 256, 512, [45, 56, 78]
+    k_dim = shape_utils.gen_int_var_min_max(ks, name="k")
+    X = Tensor(shape=[IntImm(B), k_dim, IntImm(M)], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[IntImm(B), k_dim, IntImm(N)], dtype="float16", name="input_1", is_input=True)
+    Y = _mark_output(ops.bmm_crr()(X, W))
+    module = compile_model(Y, detect_target(), WORKDIR, f"bmm_crr_dynk_{next(_counter)}")
+    for K in ks:
+        a, b = _rand((B, K, M), K), _rand((B, K, N), K + 1, K ** -0.5)
+        y = torch.empty(B, M, N, dtype=torch.float16, device="cuda")
+        module.run_with_tensors({"input_0": a.cuda(), "input_1": b.cuda()}, [y])
+        torch.testing.assert_close(y.cpu().float(), oracle.torch_bmm("crr", a, b).half().float(), atol=1e-2, rtol=1e-2)
+    module.close()
