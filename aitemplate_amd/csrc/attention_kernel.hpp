@@ -23,6 +23,8 @@
 // arguments python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:84-110).
 #pragma once
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace aitamd {
@@ -162,6 +164,12 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
             if (k0 + j < p.K) v[j] = Qb[(int64_t)q_row * p.K + k0 + j];
         }
       }
+      // a negative scale changes sides: (-Q) K^T with |scale| gives the same scaled scores, and the
+      // softmax below only ever sees a positive scale (negation is exact)
+      if (p.scale_log2e < 0.0f) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = -v[j];
+      }
       qf[ks] = v;
     }
 
@@ -269,11 +277,10 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     for (int ot = 0; ot < OT; ++ot)
 #pragma unroll
       for (int e = 0; e < 16; ++e) oacc[ot][e] = 0.0f;
-    // running extremum of the raw scores of this lane's row: the maximum, or the minimum when the
-    // scale is negative (either way the score whose scaled value is largest)
-    const bool neg_scale = p.scale_log2e < 0.0f;
-    const float m_init = neg_scale ? INFINITY : -INFINITY;
-    float m_run = m_init;
+    // running maximum of the raw scores of this lane's row (of the negated scores when the scale is
+    // negative: see the Q fragments)
+    const float c = __builtin_fabsf(p.scale_log2e);
+    float m_run = -INFINITY;
     float l_run = 0.0f;       // running sum over this lane's half of the keys
 
     // wave-loads this wave issues per tile
@@ -331,65 +338,53 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           s = Tr::mfma32(kf, qf[ks], s);
         }
         // lane holds keys nb + 8 g + 4 h + r (element 4 g + r) of query row q_row.
-        // The running maximum is kept on the raw scores (minimum when the scale is negative) and the
-        // scale is folded into the exponent: p = exp2(s * c - m * c) is one FMA and one v_exp per score.
-        // Only blocks that reach past N or touch the causal diagonal pay for masking.
-        const bool need_mask = (nb + 32 > p.N) || (p.causal && nb + 31 > m0 + wave * 32);
-        bool dead[16];
-        if (need_mask) {
+        // The running maximum is kept on the raw scores and the scale is folded into the exponent:
+        // p = exp2(s * c - m * c) is one FMA and one v_exp per score (c > 0: a negative scale was moved into
+        // the Q fragments).  Only blocks that reach past N or touch the causal diagonal pay for masking; the
+        // test is wave-uniform, so it costs one scalar branch per block.
+        const bool need_mask = (nb + 32 > p.N) || (p.causal && nb + 31 > m0 + wave_u * 32);
+        float alpha = 1.0f;
+        auto softmax_block = [&](auto masked_tag) {
+          constexpr bool MASKED = decltype(masked_tag)::value;
+          bool dead[16];
+          if constexpr (MASKED) {
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int n = nb + (e >> 2) * 8 + h * 4 + (e & 3);
-            dead[e] = (n >= p.N) || (p.causal && n > q_row);
+            for (int e = 0; e < 16; ++e) {
+              const int n = nb + (e >> 2) * 8 + h * 4 + (e & 3);
+              dead[e] = (n >= p.N) || (p.causal && n > q_row);
+            }
           }
-        }
-        float text = neg_scale ? INFINITY : -INFINITY;
-        if (need_mask) {
+          float text = -INFINITY;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) text = fmaxf(text, (MASKED && dead[e]) ? -INFINITY : s[e]);
+          text = max_across_halves(text);
+          const float m_cand = fmaxf(m_run, text);
+          // The reference point of the exponent moves only when the row maximum has grown by more than
+          // kLazyLog2 binary orders since it was last taken: until then p = exp2(s c - m c) may exceed 1 (by at
+          // most 2^kLazyLog2, harmless in fp32 sums and in the fp16 / bf16 probabilities) and the accumulators
+          // need no rescaling.  With random scores some row of a wave sets a new maximum in most blocks, so
+          // rescaling on every change costs 2 multiplies per score; this way it is rare.
+          constexpr float kLazyLog2 = 8.0f;
+          const float drift = (m_run - m_cand) * c;  // <= 0; -inf (or NaN for inf - inf) on the first live block
+          const bool move = !(drift >= -kLazyLog2);
+          const float m_new = move ? m_cand : m_run;
+          const float m_safe = __builtin_isinf(m_new) ? 0.0f : m_new;  // every key so far masked
+          alpha = !move ? 1.0f : (__builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f(drift));
+          const float mc = -m_safe * c;
+          float psum = 0.0f;
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
-            const float v = dead[e] ? m_init : s[e];
-            text = neg_scale ? fminf(text, v) : fmaxf(text, v);
-          }
-        } else if (neg_scale) {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) text = fminf(text, s[e]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) text = fmaxf(text, s[e]);
-        }
-        text = neg_scale ? min_across_halves(text) : max_across_halves(text);
-        const float m_cand = neg_scale ? fminf(m_run, text) : fmaxf(m_run, text);
-        // The reference point of the exponent moves only when the row extremum has grown by more than
-        // kLazyLog2 binary orders since it was last taken: until then p = exp2(s c - m c) may exceed 1 (by at
-        // most 2^kLazyLog2, harmless in fp32 sums and in the fp16 / bf16 probabilities) and the accumulators
-        // need no rescaling.  With random scores some row of a wave sets a new maximum in most blocks, so
-        // rescaling on every change costs 2 multiplies per score; this way it is rare.
-        constexpr float kLazyLog2 = 8.0f;
-        const float c = p.scale_log2e;
-        const float drift = (m_run - m_cand) * c;  // <= 0; -inf (or NaN for inf - inf) on the first live block
-        const bool move = !(drift >= -kLazyLog2);
-        const float m_new = move ? m_cand : m_run;
-        const float m_safe = __builtin_isinf(m_new) ? 0.0f : m_new;  // every key so far masked
-        const float alpha = !move ? 1.0f : (__builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f(drift));
-        const float mc = -m_safe * c;
-        float psum = 0.0f;
-        if (need_mask) {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const float pe = dead[e] ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc));
+            const float pe = (MASKED && dead[e]) ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc));
             s[e] = pe;
             psum += pe;
           }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc));
-            s[e] = pe;
-            psum += pe;
-          }
-        }
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
+          l_run = l_run * alpha + psum;
+          m_run = m_new;
+        };
+        if (need_mask)
+          softmax_block(std::true_type{});
+        else
+          softmax_block(std::false_type{});
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
           for (int ot = 0; ot < OT; ++ot)

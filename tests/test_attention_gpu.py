@@ -63,7 +63,7 @@ def test_bf16():
 @pytest.mark.parametrize("scale", [-0.3, 0.0])
 @pytest.mark.parametrize("causal", [False, True])
 def test_negative_and_zero_scale(scale, causal):
-    # the running extremum is kept on raw scores: a negative scale tracks the minimum instead
+    # the running maximum is kept on raw scores: a negative scale is moved into the Q fragments
     _check(8, 200, 200, 40, 40, 4, causal=causal, scale=scale, seed=9)
 
 
