@@ -232,7 +232,6 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     typedef __attribute__((address_space(3))) void lds_void;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     uint32_t d_off[L_W];  // byte offset of the lane's chunk inside K (or V) for n0 = 0; kOobOffset = always zero
-    __amdgpu_buffer_rsrc_t rk, rv;
     if constexpr (DMA) {
 #pragma unroll
       for (int i = 0; i < L_W; ++i) {
@@ -244,23 +243,21 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         const int row = idx / c1, c = idx - row * c1;
         d_off[i] = (c * 8 < dim) ? (uint32_t)((row * dim + c * 8) * 2) : kOobOffset;
       }
-      rk = make_rsrc(Kb, (uint32_t)((int64_t)p.N * p.K * 2));
-      rv = make_rsrc(Vb, (uint32_t)((int64_t)p.N * p.O * 2));
     }
+    // (the K / V choice of a wave-load is wave-uniform: scalar selects, no branches)
     auto issue_tile = [&](int n0, int stage) {
       T* dK = sK + stage * BN * KPI;
       T* dV = sV + stage * BN * VPI;
 #pragma unroll
       for (int i = 0; i < L_W; ++i) {
         const int j = wave_u + NW * i;
-        if (j >= KL + VL) continue;
-        if (j < KL) {
-          const uint32_t off = d_off[i] != kOobOffset ? d_off[i] + (uint32_t)(n0 * p.K * 2) : kOobOffset;
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_void*)(dK + j * 512), 16, off, 0, 0, 0);
-        } else {
-          const uint32_t off = d_off[i] != kOobOffset ? d_off[i] + (uint32_t)(n0 * p.O * 2) : kOobOffset;
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_void*)(dV + (j - KL) * 512), 16, off, 0, 0, 0);
-        }
+        if ((i + 1) * NW > KL + VL && j >= KL + VL) continue;  // only the last round can run past the tile
+        const bool is_k = j < KL;
+        const uint32_t off =
+            d_off[i] != kOobOffset ? d_off[i] + (uint32_t)(n0 * (is_k ? p.K : p.O) * 2) : kOobOffset;
+        T* dst = is_k ? dK + j * 512 : dV + (j - KL) * 512;
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(is_k ? Kb : Vb, (uint32_t)((int64_t)p.N * (is_k ? p.K : p.O) * 2));
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)dst, 16, off, 0, 0, 0);
       }
     };
 
