@@ -51,13 +51,25 @@ def _filter(instance_name, func_attrs, ab_alignment) -> bool:
     dtype = common.DTYPE_ID[func_attrs["inputs"][0]._attrs["dtype"]]
     lay = _kernels.LAYOUT_ID[_layout(func_attrs)[0]]
     algo = func_attrs["op_instance"][instance_name]
+    dyn_a, dyn_b = _dynamic_pitch(func_attrs)
     for key in func_attrs["exec_path"]:
         m, n, k = gemm_inverse_key_func(key)[-3:]
         lda, ldb = _pitches(func_attrs, m, n, k)
+        # a pitch that follows a dynamic dim can take any value at run time: only instances that need no
+        # pitch alignment qualify (asked for with an odd pitch)
+        lda = lda | 1 if dyn_a else lda
+        ldb = ldb | 1 if dyn_b else ldb
         if not lib.aitamd_gemm_algo_supported_layout(_epi(func_attrs), dtype, lay, algo, m, n, k, lda, ldb,
                                                      max(2, min(16, ab_alignment * 2))):
             return False
     return True
+
+
+def _dynamic_pitch(func_attrs):
+    """(A, B): True when the operand's row pitch (its innermost dim) has more than one possible value."""
+    def last_dim_is_dynamic(tensor):
+        return len(tensor._attrs["shape"][-1]._attrs["values"]) > 1
+    return last_dim_is_dynamic(func_attrs["inputs"][0]), last_dim_is_dynamic(func_attrs["inputs"][1])
 
 
 def _select_algo(func_attrs, exec_key) -> str:

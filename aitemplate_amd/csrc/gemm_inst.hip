@@ -42,7 +42,7 @@ constexpr bool kLayoutsArePermuted = AITAMD_EPI == kEpiBias;  // the bias kernel
 
 template <class Tile, bool PERM, int LAYOUT>
 struct KernelOf {
-  static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi, PERM>;
+  static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi, PERM, LAYOUT>;
 };
 template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, bool PERM, int LAYOUT>
 struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, PERM, LAYOUT> {
@@ -58,6 +58,12 @@ struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS>, PERM, LAYOUT> {
 template <class Tile>
 struct LayoutMask {
   static constexpr int value = 1;
+};
+// the element-wide loads take every layout: the instance of last resort for pitches and K that the
+// 16-byte loads cannot take
+template <int BM, int BN, int BK, int WM, int WN>
+struct LayoutMask<GemmTile<BM, BN, BK, WM, WN, 1>> {
+  static constexpr int value = kLayoutBits;
 };
 template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
 struct LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>> {
@@ -173,7 +179,7 @@ const GemmAlgo kAlgos[] = {
    BM, BN, BK, GemmTile<BM, BN, BK, WM, WN, KV>::NT, KV, GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes, \
    staged_wgs_per_cu(BM, BN, GemmTile<BM, BN, BK, WM, WN, KV>::NT,                                  \
                      GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes),                                  \
-   0, 1, &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
+   0, LayoutMask<GemmTile<BM, BN, BK, WM, WN, KV>>::value, &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
 #define AITAMD_GEMM_TILE_DMA(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX)                                 \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
    "_c" #AUX,                                                                                              \

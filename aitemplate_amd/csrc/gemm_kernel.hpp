@@ -126,8 +126,12 @@ AITAMD_DEVICE int lds_chunk_elem(int row, int chunk) {
   return row * Tile::BK + ((chunk ^ swz) << 3);
 }
 
-template <class T, class Tile, class Epi, bool PERM = false>
+// LAYOUT as in gemm_rcr_dma_kernel (bit 1: A stored [K, M]; bit 0: B stored [K, N]); the element-wide
+// loads (KVEC = 1) take any layout, pitch and alignment: the instance of last resort.
+template <class T, class Tile, class Epi, bool PERM = false, int LAYOUT = 0>
 __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) {
+  static_assert(LAYOUT == 0 || Tile::KVEC == 1, "only the element-wide loads read operands that are not K-contiguous");
+  constexpr bool A_T = (LAYOUT & 2) != 0, B_T = (LAYOUT & 1) != 0;
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int BM = Tile::BM, BN = Tile::BN, BK = Tile::BK;
@@ -162,13 +166,17 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
 #pragma unroll
   for (int i = 0; i < A_IT; ++i) {
     const int row = ld_row + i * Tile::ROWS_PER_PASS;
-    a_off[i] = (uint32_t)(((int64_t)row * p.lda + ld_chunk * 8) * 2);
+    // a transposed operand: element (row, k) lies at k * pitch + row; rows past the tile edge are masked here
+    // because they are not past the end of the buffer
+    a_off[i] = A_T ? (row < rows_a ? (uint32_t)((ld_chunk * 8 * p.lda + row) * 2) : kOobOffset)
+                   : (uint32_t)(((int64_t)row * p.lda + ld_chunk * 8) * 2);
     a_st[i] = lds_chunk_elem<Tile>(row, ld_chunk);
   }
 #pragma unroll
   for (int i = 0; i < B_IT; ++i) {
     const int row = ld_row + i * Tile::ROWS_PER_PASS;
-    b_off[i] = (uint32_t)(((int64_t)row * p.ldb + ld_chunk * 8) * 2);
+    b_off[i] = B_T ? (row < rows_b ? (uint32_t)((ld_chunk * 8 * p.ldb + row) * 2) : kOobOffset)
+                   : (uint32_t)(((int64_t)row * p.ldb + ld_chunk * 8) * 2);
     b_st[i] = lds_chunk_elem<Tile>(row, ld_chunk);
   }
 
@@ -184,10 +192,12 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
   const int k_tiles = (p.K + BK - 1) / BK;
 
   {
-    const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)batch * p.sa + (int64_t)m0 * p.lda;
-    const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)batch * p.sb + (int64_t)n0 * p.ldb;
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ab, clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2));
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
+    const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)batch * p.sa + (A_T ? (int64_t)m0 : (int64_t)m0 * p.lda);
+    const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)batch * p.sb + (B_T ? (int64_t)n0 : (int64_t)n0 * p.ldb);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(
+        Ab, clamp_records((A_T ? ((int64_t)p.K - 1) * p.lda + rows_a : ((int64_t)rows_a - 1) * p.lda + p.K) * 2));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(
+        Bb, clamp_records((B_T ? ((int64_t)p.K - 1) * p.ldb + rows_b : ((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
 
     u32x4 ga[A_IT], gb[B_IT];
 
@@ -200,7 +210,7 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
         for (int i = 0; i < B_IT; ++i) gb[i] = buffer_load_16B(rb, b_off[i] + kadd);
       } else {
         constexpr int PIECES = 8 / KVEC;
-        auto load_pieces = [&](const __amdgpu_buffer_rsrc_t& r, uint32_t base) {
+        auto load_pieces = [&](const __amdgpu_buffer_rsrc_t& r, uint32_t base, bool transposed, int64_t pitch) {
           union {
             u32x4 v;
             uint16_t s[8];
@@ -209,7 +219,8 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
 #pragma unroll
           for (int j = 0; j < PIECES; ++j) {
             const int ke = k0 + ld_chunk * 8 + j * KVEC;
-            const uint32_t off = (ke < p.K) ? base + (uint32_t)((k0 + j * KVEC) * 2) : kOobOffset;
+            const uint32_t step = transposed ? (uint32_t)((k0 + j * KVEC) * pitch * 2) : (uint32_t)((k0 + j * KVEC) * 2);
+            const uint32_t off = (ke < p.K && base != kOobOffset) ? base + step : kOobOffset;
             if constexpr (KVEC == 4) {
               const u32x2 t = buffer_load_8B(r, off);
               u.w[2 * j] = t.x;
@@ -223,9 +234,9 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
           return u.v;
         };
 #pragma unroll
-        for (int i = 0; i < A_IT; ++i) ga[i] = load_pieces(ra, a_off[i]);
+        for (int i = 0; i < A_IT; ++i) ga[i] = load_pieces(ra, a_off[i], A_T, p.lda);
 #pragma unroll
-        for (int i = 0; i < B_IT; ++i) gb[i] = load_pieces(rb, b_off[i]);
+        for (int i = 0; i < B_IT; ++i) gb[i] = load_pieces(rb, b_off[i], B_T, p.ldb);
       }
     };
 

@@ -144,7 +144,8 @@ AITAMD_API int aitamd_bmm_rcr(int dtype, int algo,
  *   AITAMD_LAYOUT_CCR: A [B, K, M], B [B, N, K]     AITAMD_LAYOUT_CRR: A [B, K, M], B [B, K, N]
  * lda / ldb are the row pitches of the matrices as stored, the strides are per batch (0 broadcasts).  d1 = 0
  * stores plainly with ldc / stride_c; d1 > 0 stores [B/d1, M, d1, N] as aitamd_bmm_rcr_permute does (ldc and
- * stride_c are ignored).  A transposed operand needs a row pitch that is a multiple of 8 elements.
+ * stride_c are ignored).  A transposed operand whose row pitch is not a multiple of 8 elements is served by the
+ * instance with element-wide loads only.
  * Replaces the DeviceBatchedGemmXdl / DeviceGemm instances behind bmm_rrr, bmm_ccr, bmm_crr, gemm_rrr and
  * bmm_rrr_permute (python/aitemplate/backend/rocm/gemm/bmm_rrr.py, bmm_ccr.py, bmm_crr.py, gemm_rrr.py,
  * bmm_rrr_permute.py; layouts in backend/rocm/gemm/layout.py). */
