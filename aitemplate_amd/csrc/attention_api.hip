@@ -1,4 +1,5 @@
 // C ABI launcher of the fused attention kernel (bmm_softmax_bmm_permute).
+#include <cstdlib>
 #include <mutex>
 
 #include "../../include/aitemplate_amd_kernels.h"
@@ -10,20 +11,28 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 
-// WIDE: eight waves (256 query rows) share each K / V tile and four LDS stages keep three tiles in
-// flight; otherwise four waves, two stages and two workgroups per CU.
-template <int KS, int OT, bool WIDE>
+// MODE 0: four waves (128 query rows), two LDS stages, two workgroups per CU.
+// MODE 1: eight waves (256 query rows) share each K / V tile and four LDS stages keep three tiles in flight.
+// MODE 2: as 1 with two groups of eight waves that take alternate tiles (sixteen waves per CU).
+template <int KS, int OT, int MODE>
 struct TileOf {
   using type = AttnTile<KS, OT>;
 };
 template <int KS, int OT>
-struct TileOf<KS, OT, true> {
+struct TileOf<KS, OT, 1> {
   using type = AttnTile<KS, OT, ((16 * KS + 32 * OT) <= 128 ? 128 : 64), 8, 4>;
 };
+template <int KS, int OT>
+struct TileOf<KS, OT, 2> {
+  // (two groups only where the merge fits the ring's memory: the small head dims this mode is chosen for)
+  static constexpr bool kFits =
+      (16 * KS + 32 * OT) <= 112 && (16 * OT + 2) * 8 * 64 * 4 <= TileOf<KS, OT, 1>::type::kLdsBytes;
+  using type = AttnTile<KS, OT, ((16 * KS + 32 * OT) <= 128 ? 128 : 64), 8, 4, kFits ? 2 : 1>;
+};
 
-template <class T, int KS, int OT, bool VEC, bool DMA, bool WIDE>
+template <class T, int KS, int OT, bool VEC, bool DMA, int MODE>
 hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
-  using Tile = typename TileOf<KS, OT, WIDE>::type;
+  using Tile = typename TileOf<KS, OT, MODE>::type;
   auto kernel = attention_kernel<T, Tile, VEC, DMA>;
   static std::once_flag once[kMaxDevices];
   int dev = 0;
@@ -43,10 +52,10 @@ hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
 
 typedef hipError_t (*AttnLaunch)(const AttnParams&, hipStream_t);
 
-template <class T, bool VEC, bool DMA, bool WIDE>
+template <class T, bool VEC, bool DMA, int MODE>
 AttnLaunch pick(int ks, int ot) {
 #define AITAMD_ATTN_CASE(KS, OT) \
-  if (ks <= KS && ot <= OT) return &launch_attention<T, KS, OT, VEC, DMA, WIDE>;
+  if (ks <= KS && ot <= OT) return &launch_attention<T, KS, OT, VEC, DMA, MODE>;
   // smallest padded head dims first; (K <= 16 KS, O <= 32 OT)
   AITAMD_ATTN_CASE(2, 1)
   AITAMD_ATTN_CASE(3, 2)
@@ -106,15 +115,25 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
   // 256-row workgroups for small head dims (where re-streaming K / V per 128 query rows costs most; measured
   // slower at head dims 64 and 128) once there are enough of them to fill the CUs
   const bool wide = dma && (16 * ks + 32 * ot) <= 112 && ((M + 255) / 256) * B >= 256;
+  // two wave groups pay when a CU holds one workgroup anyway: measured 4.5 % faster with 256 workgroups
+  // (16 heads x 4096 rows, head dim 40), 2 % slower with 512
+  int mode = wide ? (((M + 255) / 256) * B <= 256 ? 2 : 1) : 0;
+  // AITAMD_ATTN_MODE=0|1|2 forces a variant where the shape allows it (a test and measurement knob)
+  if (const char* forced = getenv("AITAMD_ATTN_MODE")) {
+    const int m = atoi(forced);
+    if (m >= 0 && m <= 2 && dma && (16 * ks + 32 * ot) <= 112) mode = m;
+  }
   AttnLaunch fn = nullptr;
   if (dtype == 0)
-    fn = wide ? pick<f16, true, true, true>(ks, ot)
-              : (dma ? pick<f16, true, true, false>(ks, ot)
-                     : (vec ? pick<f16, true, false, false>(ks, ot) : pick<f16, false, false, false>(ks, ot)));
+    fn = mode == 2 ? pick<f16, true, true, 2>(ks, ot)
+                   : (mode == 1 ? pick<f16, true, true, 1>(ks, ot)
+                                : (dma ? pick<f16, true, true, 0>(ks, ot)
+                                       : (vec ? pick<f16, true, false, 0>(ks, ot) : pick<f16, false, false, 0>(ks, ot))));
   else
-    fn = wide ? pick<bf16, true, true, true>(ks, ot)
-              : (dma ? pick<bf16, true, true, false>(ks, ot)
-                     : (vec ? pick<bf16, true, false, false>(ks, ot) : pick<bf16, false, false, false>(ks, ot)));
+    fn = mode == 2 ? pick<bf16, true, true, 2>(ks, ot)
+                   : (mode == 1 ? pick<bf16, true, true, 1>(ks, ot)
+                                : (dma ? pick<bf16, true, true, 0>(ks, ot)
+                                       : (vec ? pick<bf16, true, false, 0>(ks, ot) : pick<bf16, false, false, 0>(ks, ot))));
   if (!fn) return fail("aitamd_bmm_softmax_bmm_permute: no instance for K=%lld O=%lld", (long long)K, (long long)O);
   const hipError_t e = fn(p, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail("aitamd_bmm_softmax_bmm_permute: launch failed: %s", hipGetErrorString(e));

@@ -41,16 +41,18 @@ struct AttnParams {
 
 // NW_ waves (32 query rows each) share the K / V tiles; NS_ LDS stages.  The register-staged
 // loaders use two stages; the direct-to-LDS path keeps NS_ - 1 tiles in flight.
-template <int KS_, int OT_, int BN_ = ((16 * KS_ + 32 * OT_) <= 112 ? 128 : 64), int NW_ = 4, int NS_ = 2>
+// NG_ groups of NW_ waves each take every NG_-th tile of the same query rows and merge their running
+// sums at the end: twice the waves per SIMD for the same K / V traffic.
+template <int KS_, int OT_, int BN_ = ((16 * KS_ + 32 * OT_) <= 112 ? 128 : 64), int NW_ = 4, int NS_ = 2, int NG_ = 1>
 struct AttnTile {
   static constexpr int KS = KS_;          // K padded to 16 * KS
   static constexpr int OT = OT_;          // O padded to 32 * OT
   static constexpr int KP = 16 * KS;
   static constexpr int OP = 32 * OT;
-  static constexpr int NW = NW_, NS = NS_;
+  static constexpr int NW = NW_, NS = NS_, NG = NG_;
   static constexpr int BM = 32 * NW;      // query rows per workgroup
   static constexpr int BN = BN_;          // keys per LDS tile: 128 while two workgroups still fit one CU's LDS
-  static constexpr int NT = 64 * NW;
+  static constexpr int NT = 64 * NW * NG;
   static constexpr int K_PITCH = KP + 8;  // halves; keeps 16 consecutive rows on distinct banks
   static constexpr int V_PITCH = OP + 8;
   static constexpr int K_CHUNKS = BN * KP / 8;  // 16-byte chunks per tile (pads included)
@@ -59,6 +61,8 @@ struct AttnTile {
   static constexpr int V_IT = (V_CHUNKS + NT - 1) / NT;
   static constexpr int kLdsBytes = NS * BN * (K_PITCH + V_PITCH) * 2;
   static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
+  static_assert(NG == 1 || (NS % NG == 0 && NS >= 2 * NG), "the groups' tiles and the next ones in flight need a stage each");
+  static_assert(NG == 1 || (16 * OT + 2) * NW * 64 * 4 <= kLdsBytes, "the merge goes through the ring's memory");
 };
 
 // LDS transpose read: 4 x 16-bit per lane, gathered across the 16 lanes of a block
@@ -125,7 +129,8 @@ template <class T, class Tile, bool VEC, bool DMA = false>
 __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_kernel(const AttnParams p) {
   static_assert(!DMA || VEC, "the direct-to-LDS path needs 16-byte chunks");
   static_assert(DMA || Tile::NS == 2, "the register-staged loaders double-buffer");
-  constexpr int NS = Tile::NS, NW = Tile::NW;
+  static_assert(DMA || Tile::NG == 1, "wave groups need the direct-to-LDS loader");
+  constexpr int NS = Tile::NS, NW = Tile::NW, NG = Tile::NG, NWT = NW * NG;
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
   using vec4 = typename Tr::vec4;
@@ -138,7 +143,9 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave_all = tid >> 6;
+  const int grp = __builtin_amdgcn_readfirstlane(wave_all / NW);  // which tiles this wave takes
+  const int wave = wave_all % NW;                                 // which 32 query rows
   const int r32 = lane & 31;
   const int h = lane >> 5;
   const int m0 = blockIdx.x * Tile::BM;
@@ -226,16 +233,17 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     // ---- direct-to-LDS tile loader: the KL + VL wave-loads of a tile are dealt round-robin to the waves
     constexpr int KC1 = KP / 8 + 1, VC1 = OP / 8 + 1;        // chunks per LDS row, pad chunk included
     constexpr int KL = BN * KC1 / 64, VL = BN * VC1 / 64;     // wave-loads per K / V tile
-    constexpr int L_W = (KL + VL + NW - 1) / NW;
+    constexpr int L_W = (KL + VL + NWT - 1) / NWT;
     static_assert((BN * KC1) % 64 == 0 && (BN * VC1) % 64 == 0, "tiles must be whole wave-loads");
     static_assert(Tile::K_PITCH == KC1 * 8 && Tile::V_PITCH == VC1 * 8, "LDS rows are the chunks of a row plus one");
     typedef __attribute__((address_space(3))) void lds_void;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int wave_ld = __builtin_amdgcn_readfirstlane(wave_all);  // the loads are dealt over all waves
     uint32_t d_off[L_W];  // byte offset of the lane's chunk inside K (or V) for n0 = 0; kOobOffset = always zero
     if constexpr (DMA) {
 #pragma unroll
       for (int i = 0; i < L_W; ++i) {
-        const int j = wave_u + NW * i;
+        const int j = wave_ld + NWT * i;
         const bool is_k = j < KL;
         const int idx = (is_k ? j : j - KL) * 64 + lane;
         const int c1 = is_k ? KC1 : VC1;
@@ -250,8 +258,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
       T* dV = sV + stage * BN * VPI;
 #pragma unroll
       for (int i = 0; i < L_W; ++i) {
-        const int j = wave_u + NW * i;
-        if ((i + 1) * NW > KL + VL && j >= KL + VL) continue;  // only the last round can run past the tile
+        const int j = wave_ld + NWT * i;
+        if ((i + 1) * NWT > KL + VL && j >= KL + VL) continue;  // only the last round can run past the tile
         const bool is_k = j < KL;
         const uint32_t off =
             d_off[i] != kOobOffset ? d_off[i] + (uint32_t)(n0 * (is_k ? p.K : p.O) * 2) : kOobOffset;
@@ -281,8 +289,13 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     float l_run = 0.0f;       // running sum over this lane's half of the keys
 
     // wave-loads this wave issues per tile
-    const int my_loads = (KL + VL - wave_u + NW - 1) / NW;
-    if constexpr (DMA) {
+    const int my_loads = (KL + VL - wave_ld + NWT - 1) / NWT;
+    if constexpr (DMA && NG > 1) {
+      // every group's first tile; later tiles are issued one iteration ahead (see the loop)
+#pragma unroll
+      for (int g = 0; g < NG; ++g)
+        if (g < n_tiles) issue_tile(g * BN, g);
+    } else if constexpr (DMA) {
       // NS - 1 tiles in flight; tiles past the last one are all out of range (zero fill, no traffic),
       // issued all the same so that the number of loads per tile stays constant for the waits
       if (n_tiles > 0) {
@@ -305,9 +318,23 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     const int tr_col = ((lane >> 4) & 1) * 16 + (tr_i & 3) * 4;
 
     int cur = 0;
-    for (int t = 0; t < n_tiles; ++t) {
+    const int n_iters = (n_tiles + NG - 1) / NG;
+    for (int it = 0; it < n_iters; ++it) {
+      const int t = it * NG + grp;  // this wave's tile
       const bool has_next = (t + 1) < n_tiles;
-      if constexpr (DMA) {
+      if constexpr (DMA && NG > 1) {
+        // the tiles of this iteration were issued one iteration ago; past the barrier the stages of the
+        // previous iteration are free and take the next iteration's tiles
+        attn_wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          const int tn = (it + 1) * NG + g;
+          if (tn < n_tiles) issue_tile(tn * BN, tn % NS);
+        }
+        cur = t % NS;
+        if (t >= n_tiles) continue;  // the last iteration can be short of tiles
+      } else if constexpr (DMA) {
         // this wave's part of tile t has landed once only the NS - 2 younger tiles are in flight; past
         // the barrier everybody's has, and nobody reads the stage of tile t - 1 any more, so tile
         // t + NS - 1 starts landing there
@@ -414,13 +441,45 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         if (has_next) store_tiles(cur ^ 1);
         __syncthreads();
       }
-      cur = cur + 1 == NS ? 0 : cur + 1;
+      if constexpr (NG == 1) cur = cur + 1 == NS ? 0 : cur + 1;
+    }
+
+    // ---- wave groups: the other groups hand their running state to group 0 through the ring's memory
+    if constexpr (NG > 1) {
+      attn_wait_vmcnt<0>();
+      __syncthreads();  // nobody reads tiles any more and nothing is landing
+      float* xch = reinterpret_cast<float*>(smem_raw);
+      constexpr int NV = 16 * OT + 2;
+      static_assert(NG == 2, "the merge below pairs two groups");
+      if (grp == 1) {
+#pragma unroll
+        for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) xch[((ot * 16 + e) * NW + wave) * 64 + lane] = oacc[ot][e];
+        xch[((NV - 2) * NW + wave) * 64 + lane] = m_run;
+        xch[((NV - 1) * NW + wave) * 64 + lane] = l_run;
+      }
+      __syncthreads();
+      if (grp == 0) {
+        const float m1 = xch[((NV - 2) * NW + wave) * 64 + lane];
+        const float l1 = xch[((NV - 1) * NW + wave) * 64 + lane];
+        // both states are sums of exp2((s - m) c) terms for their own reference m: bring them to the larger one
+        const float m = fmaxf(m_run, m1);
+        const float a0 = __builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m) * c);
+        const float a1 = __builtin_isinf(m1) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * c);
+        l_run = l_run * a0 + l1 * a1;
+#pragma unroll
+        for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            oacc[ot][e] = oacc[ot][e] * a0 + xch[((ot * 16 + e) * NW + wave) * 64 + lane] * a1;
+      }
     }
 
     // ---- normalise and store permuted: out[b / G][m][b % G][o]
     const float l_tot = sum_across_halves(l_run);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    if (q_row < p.M) {
+    if (q_row < p.M && grp == 0) {
       T* orow = reinterpret_cast<T*>(p.out) + (((int64_t)(b / p.G) * p.M + q_row) * p.G + (b % p.G)) * p.O;
       const bool vec_ok = ((p.O & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 7) == 0);
 #pragma unroll

@@ -55,6 +55,23 @@ def test_ragged_and_odd_shapes(B, M, N, K, O, G, causal):
     _check(B, M, N, K, O, G, causal, seed=3)
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("B,M,N,K,O,G,causal,scale", [
+    (8, 300, 1000, 40, 40, 4, False, None),    # 8 key tiles: both wave groups busy
+    (8, 300, 900, 40, 40, 4, True, None),      # causal: workgroups stop at different tiles
+    (4, 100, 130, 40, 40, 2, False, -0.2),     # 2 tiles, the second ragged; negative scale
+    (4, 70, 384, 32, 32, 4, False, None),      # 3 tiles: the second group is short of one
+    (2, 40, 50, 40, 40, 2, True, None),        # a single tile: the second group has nothing to merge
+    (2, 260, 0, 40, 40, 2, False, None),       # no keys at all
+])
+def test_every_variant_of_the_small_head_dims(monkeypatch, mode, B, M, N, K, O, G, causal, scale):
+    # AITAMD_ATTN_MODE picks the variant where the shape allows it: 0 four waves, 1 eight waves, 2 two groups of
+    # eight waves that take alternate key tiles and merge their running sums at the end
+    monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+    print(f"case attention mode={mode} B={B} M={M} N={N} K={K} causal={causal} scale={scale}", flush=True)
+    _check(B, M, N, K, O, G, causal=causal, scale=scale, seed=mode + N)
+
+
 def test_bf16():
     _check(8, 200, 136, 64, 64, 4, dtype=torch.bfloat16, tol=4e-2)
     _check(8, 100, 100, 40, 40, 8, causal=True, dtype=torch.bfloat16, tol=4e-2)
