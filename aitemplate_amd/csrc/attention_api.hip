@@ -26,7 +26,7 @@ template <int KS, int OT>
 struct TileOf<KS, OT, 2> {
   // (two groups only where the merge fits the ring's memory: the small head dims this mode is chosen for)
   static constexpr bool kFits =
-      (16 * KS + 32 * OT) <= 112 && (16 * OT + 2) * 8 * 64 * 4 <= TileOf<KS, OT, 1>::type::kLdsBytes;
+      (16 * KS + 32 * OT) <= 128 && (16 * OT + 2) * 8 * 64 * 4 <= TileOf<KS, OT, 1>::type::kLdsBytes;
   using type = AttnTile<KS, OT, ((16 * KS + 32 * OT) <= 128 ? 128 : 64), 8, 4, kFits ? 2 : 1>;
 };
 
@@ -121,7 +121,7 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
   // AITAMD_ATTN_MODE=0|1|2 forces a variant where the shape allows it (a test and measurement knob)
   if (const char* forced = getenv("AITAMD_ATTN_MODE")) {
     const int m = atoi(forced);
-    if (m >= 0 && m <= 2 && dma && (16 * ks + 32 * ot) <= 112) mode = m;
+    if (m >= 0 && m <= 2 && dma && (16 * ks + 32 * ot) <= 128) mode = m;
   }
   AttnLaunch fn = nullptr;
   if (dtype == 0)

@@ -148,10 +148,24 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
   const int wave = wave_all % NW;                                 // which 32 query rows
   const int r32 = lane & 31;
   const int h = lane >> 5;
-  const int m0 = blockIdx.x * Tile::BM;
+  // Workgroup -> (query tile, batch entry).  The hardware deals consecutive workgroup ids round-robin over the
+  // 8 XCDs, each with its own L2; dealt plainly, the workgroups of one batch entry land on all of them and every
+  // L2 fetches that entry's K and V.  When the grid divides evenly, XCD x takes the x-th eighth of the
+  // (batch entry, query tile) pairs instead, so the workgroups that stream the same K / V share one L2.
+  int bx = blockIdx.x, by = blockIdx.y;
+  {
+    const int total = gridDim.x * gridDim.y;
+    if ((int)gridDim.y == p.B && (total & 7) == 0) {
+      const int id = blockIdx.x + gridDim.x * blockIdx.y;
+      const int v = (id & 7) * (total >> 3) + (id >> 3);
+      by = v / (int)gridDim.x;
+      bx = v - by * (int)gridDim.x;
+    }
+  }
+  const int m0 = bx * Tile::BM;
   const int q_row = m0 + wave * 32 + r32;  // this lane's query row
 
-  for (int b = blockIdx.y; b < p.B; b += gridDim.y) {
+  for (int b = by; b < p.B; b += gridDim.y) {
     const T* Qb = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.M * p.K;
     const T* Kb = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.N * p.K;
     const T* Vb = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.N * p.O;
