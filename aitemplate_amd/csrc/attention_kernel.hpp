@@ -85,6 +85,28 @@ struct AttnVec<bf16> {
   }
 };
 
+// acc + the 8 elements of v: four v_dot2 against (1, 1) on the packed pairs as they lie in the registers
+AITAMD_DEVICE float add_elements(f16x8 v, float acc) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  struct Quads {
+    h2 q[4];
+  };
+  const Quads u = __builtin_bit_cast(Quads, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2(u.q[i], h2{(f16)1.0f, (f16)1.0f}, acc, false);
+  return acc;
+}
+AITAMD_DEVICE float add_elements(bf16x8 v, float acc) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  struct Quads {
+    b2 q[4];
+  };
+  const Quads u = __builtin_bit_cast(Quads, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2_f32_bf16(u.q[i], b2{(bf16)1.0f, (bf16)1.0f}, acc, false);
+  return acc;
+}
+
 AITAMD_DEVICE float max_across_halves(float x) {
   // lane l and lane l^32 hold the two halves of one query row
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -382,6 +404,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         // test is wave-uniform, so it costs one scalar branch per block.
         const bool need_mask = (nb + 32 > p.N) || (p.causal && nb + 31 > m0 + wave_u * 32);
         float alpha = 1.0f;
+        vec8 pf[2];  // P^T fragments of the block's two 16-key steps
         auto softmax_block = [&](auto masked_tag) {
           constexpr bool MASKED = decltype(masked_tag)::value;
           bool dead[16];
@@ -409,14 +432,19 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           const float m_safe = __builtin_isinf(m_new) ? 0.0f : m_new;  // every key so far masked
           alpha = !move ? 1.0f : (__builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f(drift));
           const float mc = -m_safe * c;
-          float psum = 0.0f;
+          // the probabilities are rounded to the element type at once (the second product takes them so) and the
+          // row sum adds the rounded values, two per instruction
+          l_run *= alpha;
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const float pe = (MASKED && dead[e]) ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc));
-            s[e] = pe;
-            psum += pe;
+          for (int st = 0; st < 2; ++st) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const int e = st * 8 + j;
+              pf[st][j] =
+                  Tr::from_float((MASKED && dead[e]) ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc)));
+            }
+            l_run = add_elements(pf[st], l_run);
           }
-          l_run = l_run * alpha + psum;
           m_run = m_new;
         };
         if (need_mask)
@@ -432,9 +460,6 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         // ---- O^T += V^T P^T over the block's two 16-key steps
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
-          vec8 pf;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) pf[j] = Tr::from_float(s[st * 8 + j]);
 #pragma unroll
           for (int ot = 0; ot < OT; ++ot) {
             const T* vb = cV + (blk * 32 + st * 16 + h * 4 + tr_row) * VPI + ot * 32 + tr_col;
@@ -446,7 +471,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
               vf[j] = lo[j];
               vf[4 + j] = hi[j];
             }
-            oacc[ot] = Tr::mfma32(vf, pf, oacc[ot]);
+            oacc[ot] = Tr::mfma32(vf, pf[st], oacc[ot]);
           }
         }
       }
