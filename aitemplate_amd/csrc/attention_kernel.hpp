@@ -27,6 +27,10 @@
 
 #include "common.hpp"
 
+#ifndef AITAMD_ATTN_KB
+#define AITAMD_ATTN_KB(KS, OT) (((KS) + 2 * (OT)) <= 7 ? 2 : 1)
+#endif
+
 namespace aitamd {
 
 struct AttnParams {
@@ -353,6 +357,11 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     const int tr_row = tr_i >> 2;
     const int tr_col = ((lane >> 4) & 1) * 16 + (tr_i & 3) * 4;
 
+    // 32-key sub-blocks per softmax step: two for head dims up to 48, which halves the per-step work (exchange
+    // across halves, rescale test, branches) per key: 3.7 % faster at head dim 40; at 64 the 16 extra
+    // registers cost a resident workgroup and it measures equal, so one there
+    constexpr int KB = AITAMD_ATTN_KB(KS, OT);
+    static_assert(BN % (32 * KB) == 0, "a tile is whole blocks");
     int cur = 0;
     const int n_iters = (n_tiles + NG - 1) / NG;
     for (int it = 0; it < n_iters; ++it) {
@@ -384,40 +393,48 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
       const T* cV = sV + cur * BN * VPI;
 
 #pragma unroll
-      for (int blk = 0; blk < BN / 32; ++blk) {
-        const int nb = t * BN + blk * 32;  // first key of this 32-key block
-        // ---- S^T block: rows = keys, columns = this wave's 32 query rows
+      for (int blk = 0; blk < BN / (32 * KB); ++blk) {
+        const int nb = t * BN + blk * 32 * KB;  // first key of this block of KB x 32 keys
+        // ---- S^T sub-blocks: rows = keys, columns = this wave's 32 query rows
         // (issuing the next block's product ahead of this block's softmax was measured: no gain at
         // head dim 40 and a quarter slower at head dim 64, where the extra live accumulator costs more)
-        f32x16 s;
+        f32x16 s[KB];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = 0.0f;
+        for (int kb = 0; kb < KB; ++kb) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const vec8 kf = *reinterpret_cast<const vec8*>(cK + (blk * 32 + r32) * KPI + ks * 16 + h * 8);
-          s = Tr::mfma32(kf, qf[ks], s);
+          for (int e = 0; e < 16; ++e) s[kb][e] = 0.0f;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const vec8 kf =
+                *reinterpret_cast<const vec8*>(cK + ((blk * KB + kb) * 32 + r32) * KPI + ks * 16 + h * 8);
+            s[kb] = Tr::mfma32(kf, qf[ks], s[kb]);
+          }
         }
-        // lane holds keys nb + 8 g + 4 h + r (element 4 g + r) of query row q_row.
+        // lane holds keys nb + 32 kb + 8 g + 4 h + r (element 4 g + r of sub-block kb) of query row q_row.
         // The running maximum is kept on the raw scores and the scale is folded into the exponent:
         // p = exp2(s * c - m * c) is one FMA and one v_exp per score (c > 0: a negative scale was moved into
         // the Q fragments).  Only blocks that reach past N or touch the causal diagonal pay for masking; the
         // test is wave-uniform, so it costs one scalar branch per block.
-        const bool need_mask = (nb + 32 > p.N) || (p.causal && nb + 31 > m0 + wave_u * 32);
+        const bool need_mask = (nb + 32 * KB > p.N) || (p.causal && nb + 32 * KB - 1 > m0 + wave_u * 32);
         float alpha = 1.0f;
-        vec8 pf[2];  // P^T fragments of the block's two 16-key steps
+        vec8 pf[2 * KB];  // P^T fragments of the block's 16-key steps
         auto softmax_block = [&](auto masked_tag) {
           constexpr bool MASKED = decltype(masked_tag)::value;
-          bool dead[16];
+          bool dead[KB][16];
           if constexpr (MASKED) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-              const int n = nb + (e >> 2) * 8 + h * 4 + (e & 3);
-              dead[e] = (n >= p.N) || (p.causal && n > q_row);
-            }
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) {
+                const int n = nb + kb * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+                dead[kb][e] = (n >= p.N) || (p.causal && n > q_row);
+              }
           }
           float text = -INFINITY;
 #pragma unroll
-          for (int e = 0; e < 16; ++e) text = fmaxf(text, (MASKED && dead[e]) ? -INFINITY : s[e]);
+          for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) text = fmaxf(text, (MASKED && dead[kb][e]) ? -INFINITY : s[kb][e]);
           text = max_across_halves(text);
           const float m_cand = fmaxf(m_run, text);
           // The reference point of the exponent moves only when the row maximum has grown by more than
@@ -436,12 +453,12 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           // row sum adds the rounded values, two per instruction
           l_run *= alpha;
 #pragma unroll
-          for (int st = 0; st < 2; ++st) {
+          for (int st = 0; st < 2 * KB; ++st) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-              const int e = st * 8 + j;
-              pf[st][j] =
-                  Tr::from_float((MASKED && dead[e]) ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c, mc)));
+              const int kb = st >> 1, e = (st & 1) * 8 + j;
+              pf[st][j] = Tr::from_float(
+                  (MASKED && dead[kb][e]) ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][e], c, mc)));
             }
             l_run = add_elements(pf[st], l_run);
           }
@@ -457,12 +474,12 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[ot][e] *= alpha;
         }
-        // ---- O^T += V^T P^T over the block's two 16-key steps
+        // ---- O^T += V^T P^T over the block's 16-key steps
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
+        for (int st = 0; st < 2 * KB; ++st) {
 #pragma unroll
           for (int ot = 0; ot < OT; ++ot) {
-            const T* vb = cV + (blk * 32 + st * 16 + h * 4 + tr_row) * VPI + ot * 32 + tr_col;
+            const T* vb = cV + (blk * KB * 32 + st * 16 + h * 4 + tr_row) * VPI + ot * 32 + tr_col;
             const vec4 lo = AttnVec<T>::tr_read(vb);
             const vec4 hi = AttnVec<T>::tr_read(vb + 8 * VPI);
             vec8 vf;
