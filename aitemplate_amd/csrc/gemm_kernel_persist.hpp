@@ -107,7 +107,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 #pragma unroll
   for (int i = 0; i < L; ++i) {
     const int j = wave + i * Tile::NW;
-    const bool is_a = j < Tile::A_LOADS;
+    // (with A_LOADS a multiple of the wave count, whether load i fetches A or B is the same for every wave)
+    const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
     const int row = (is_a ? j : j - Tile::A_LOADS) * Tile::ROWS_PER_LOAD + l_row;
     const int chunk = l_slot ^ ((row / Tile::RPW) % Tile::CPR);
     l_off[i] = (uint32_t)(((int64_t)row * (is_a ? p.lda : p.ldb) + chunk * 8) * 2);
@@ -163,7 +164,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       const int j = wave + i * Tile::NW;
       const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + (uint32_t)(k0 * 2) : kOobOffset;
       T* dst = sbase + j * 512;  // 1 KiB per wave-load; A blocks then B blocks
-      if (j < Tile::A_LOADS)
+      const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
+      if (is_a)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)dst, 16, off, 0, 0, 0);
       else
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)dst, 16, off, 0, 0, 0);
