@@ -189,7 +189,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
 #pragma unroll
   for (int i = 0; i < L_IT; ++i) {
     const int j = wave + i * Tile::NW;
-    const bool is_a = j < Tile::A_LOADS;
+    // (with A_LOADS a multiple of the wave count, whether load i fetches A or B is the same for every wave)
+    const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
     const int64_t ld = is_a ? p.lda : p.ldb;
     if ((is_a && A_T) || (!is_a && B_T)) {
       // 1 KiB of the operand's slab = 512 / BX whole k-rows of BX elements
@@ -259,7 +260,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
         const uint32_t step = (A_T || B_T) ? (uint32_t)k0 * l_kbytes[i] : (uint32_t)(k0 * 2);
         const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + step : kOobOffset;
         T* dst = sbase + j * 512;  // 1 KiB = 512 elements per wave-load; A blocks then B blocks
-        if (j < Tile::A_LOADS)
+        const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
+        if (is_a)
           __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)dst, 16, off, 0, 0, AUX);
         else
           __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)dst, 16, off, 0, 0, AUX);
