@@ -2,8 +2,9 @@
 // folded into the store (bmm_softmax_bmm_permute), gfx950.
 //
 // The score matrix never leaves the chip.  One wave owns 32 query rows and walks
-// the keys/values in blocks of 32; a workgroup of 4 waves shares each 64- or
-// 128-row K / V tile through LDS.
+// the keys/values in blocks of 32 (64 for the smallest head dims); a workgroup of 4 or
+// 8 waves shares each 64- or 128-row K / V tile through LDS, and the 16-wave form runs
+// two such groups on alternate tiles of the same rows and merges them at the end.
 //
 //  * S^T = K Q^T is computed with v_mfma_f32_32x32x16 (K tile rows as the A
 //    operand, the wave's Q rows - kept in registers for the whole kernel - as
@@ -115,10 +116,6 @@ AITAMD_DEVICE float max_across_halves(float x) {
   // lane l and lane l^32 hold the two halves of one query row
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-AITAMD_DEVICE float min_across_halves(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fminf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 AITAMD_DEVICE float sum_across_halves(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
