@@ -30,6 +30,14 @@ struct TileOf<KS, OT, 2> {
   using type = AttnTile<KS, OT, ((16 * KS + 32 * OT) <= 128 ? 128 : 64), 8, 4, kFits ? 2 : 1>;
 };
 
+// MODE 3: as 0 with two groups of four waves on alternate tiles and four LDS stages: for grids that leave CUs idle.
+template <int KS, int OT>
+struct TileOf<KS, OT, 3> {
+  using Base = AttnTile<KS, OT>;
+  static constexpr bool kFits = (16 * OT + 2) * 4 * 64 * 4 <= 2 * Base::kLdsBytes && 2 * Base::kLdsBytes <= 160 * 1024;
+  using type = AttnTile<KS, OT, Base::BN, 4, kFits ? 4 : 2, kFits ? 2 : 1>;
+};
+
 template <class T, int KS, int OT, bool VEC, bool DMA, int MODE>
 hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
   using Tile = typename TileOf<KS, OT, MODE>::type;
@@ -118,19 +126,25 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
   // two wave groups pay when a CU holds one workgroup anyway: measured 4.5 % faster with 256 workgroups
   // (16 heads x 4096 rows, head dim 40), 2 % slower with 512
   int mode = wide ? (((M + 255) / 256) * B <= 256 ? 2 : 1) : 0;
-  // AITAMD_ATTN_MODE=0|1|2 forces a variant where the shape allows it (a test and measurement knob)
+  // grids of 128-row workgroups that leave CUs idle take the two-group form of those too: 8-19 % faster from 48 to
+  // 256 workgroups (head dims 40 and 64), 7 % slower at 384
+  if (mode == 0 && dma && ((M + 127) / 128) * B <= 256) mode = 3;
+  // AITAMD_ATTN_MODE=0|1|2|3 forces a variant where the shape allows it (a test and measurement knob)
   if (const char* forced = getenv("AITAMD_ATTN_MODE")) {
     const int m = atoi(forced);
     if (m >= 0 && m <= 2 && dma && (16 * ks + 32 * ot) <= 128) mode = m;
+    if (m == 3 && dma) mode = 3;
   }
   AttnLaunch fn = nullptr;
   if (dtype == 0)
-    fn = mode == 2 ? pick<f16, true, true, 2>(ks, ot)
+    fn = mode == 3 ? pick<f16, true, true, 3>(ks, ot)
+       : mode == 2 ? pick<f16, true, true, 2>(ks, ot)
                    : (mode == 1 ? pick<f16, true, true, 1>(ks, ot)
                                 : (dma ? pick<f16, true, true, 0>(ks, ot)
                                        : (vec ? pick<f16, true, false, 0>(ks, ot) : pick<f16, false, false, 0>(ks, ot))));
   else
-    fn = mode == 2 ? pick<bf16, true, true, 2>(ks, ot)
+    fn = mode == 3 ? pick<bf16, true, true, 3>(ks, ot)
+       : mode == 2 ? pick<bf16, true, true, 2>(ks, ot)
                    : (mode == 1 ? pick<bf16, true, true, 1>(ks, ot)
                                 : (dma ? pick<bf16, true, true, 0>(ks, ot)
                                        : (vec ? pick<bf16, true, false, 0>(ks, ot) : pick<bf16, false, false, 0>(ks, ot))));

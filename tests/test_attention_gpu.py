@@ -55,7 +55,7 @@ def test_ragged_and_odd_shapes(B, M, N, K, O, G, causal):
     _check(B, M, N, K, O, G, causal, seed=3)
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
 @pytest.mark.parametrize("B,M,N,K,O,G,causal,scale", [
     (8, 300, 1000, 40, 40, 4, False, None),    # 8 key tiles: both wave groups busy
     (8, 300, 900, 40, 40, 4, True, None),      # causal: workgroups stop at different tiles
@@ -65,8 +65,8 @@ def test_ragged_and_odd_shapes(B, M, N, K, O, G, causal):
     (2, 260, 0, 40, 40, 2, False, None),       # no keys at all
 ])
 def test_every_variant_of_the_small_head_dims(monkeypatch, mode, B, M, N, K, O, G, causal, scale):
-    # AITAMD_ATTN_MODE picks the variant where the shape allows it: 0 four waves, 1 eight waves, 2 two groups of
-    # eight waves that take alternate key tiles and merge their running sums at the end
+    # AITAMD_ATTN_MODE picks the variant where the shape allows it: 0 four waves, 1 eight waves, 2 (3) two groups of
+    # eight (four) waves that take alternate key tiles and merge their running sums at the end
     monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
     print(f"case attention mode={mode} B={B} M={M} N={N} K={K} causal={causal} scale={scale}", flush=True)
     _check(B, M, N, K, O, G, causal=causal, scale=scale, seed=mode + N)

@@ -87,7 +87,7 @@ def test_attention_random_shapes(monkeypatch):
         causal = rng.random() < 0.4
         dtype = torch.float16 if rng.random() < 0.7 else torch.bfloat16
         scale = rng.choice([K ** -0.5, K ** -0.5, 0.3, -0.2, 1.0 / 8])
-        mode = rng.choice([None, 0, 1, 2])  # kernel variant, where the head dims allow the choice
+        mode = rng.choice([None, 0, 1, 2, 3])  # kernel variant, where the head dims allow the choice
         if mode is None:
             monkeypatch.delenv("AITAMD_ATTN_MODE", raising=False)
         else:
