@@ -18,16 +18,29 @@ template <int KS, int OT, int MODE>
 struct TileOf {
   using type = AttnTile<KS, OT>;
 };
+constexpr int wide_bn(int ks, int ot) { return (16 * ks + 32 * ot) <= 128 ? 128 : 64; }
+constexpr bool wide_fits(int ks, int ot) {  // four stages of the wide tile within the LDS
+  return 4 * wide_bn(ks, ot) * (16 * ks + 8 + 32 * ot + 8) * 2 <= 160 * 1024;
+}
+template <int KS, int OT, bool FITS = wide_fits(KS, OT)>
+struct WideTile {  // head dims too large for the wide forms keep the four-wave tile
+  using one = AttnTile<KS, OT>;
+  using two = AttnTile<KS, OT>;
+};
+template <int KS, int OT>
+struct WideTile<KS, OT, true> {
+  using one = AttnTile<KS, OT, wide_bn(KS, OT), 8, 4>;
+  // (two groups only where the merge fits the ring's memory: the small head dims this mode is chosen for)
+  static constexpr bool kMergeFits = (16 * KS + 32 * OT) <= 128 && (16 * OT + 2) * 8 * 64 * 4 <= one::kLdsBytes;
+  using two = AttnTile<KS, OT, wide_bn(KS, OT), 8, 4, kMergeFits ? 2 : 1>;
+};
 template <int KS, int OT>
 struct TileOf<KS, OT, 1> {
-  using type = AttnTile<KS, OT, ((16 * KS + 32 * OT) <= 128 ? 128 : 64), 8, 4>;
+  using type = typename WideTile<KS, OT>::one;
 };
 template <int KS, int OT>
 struct TileOf<KS, OT, 2> {
-  // (two groups only where the merge fits the ring's memory: the small head dims this mode is chosen for)
-  static constexpr bool kFits =
-      (16 * KS + 32 * OT) <= 128 && (16 * OT + 2) * 8 * 64 * 4 <= TileOf<KS, OT, 1>::type::kLdsBytes;
-  using type = AttnTile<KS, OT, ((16 * KS + 32 * OT) <= 128 ? 128 : 64), 8, 4, kFits ? 2 : 1>;
+  using type = typename WideTile<KS, OT>::two;
 };
 
 // MODE 3: as 0 with two groups of four waves on alternate tiles and four LDS stages: for grids that leave CUs idle.
@@ -71,6 +84,7 @@ AttnLaunch pick(int ks, int ot) {
   AITAMD_ATTN_CASE(4, 4)
   AITAMD_ATTN_CASE(6, 3)
   AITAMD_ATTN_CASE(8, 4)
+  AITAMD_ATTN_CASE(10, 5)  // head dim 160: the deepest attention of Stable Diffusion v1 (1280 channels, 8 heads)
 #undef AITAMD_ATTN_CASE
   return nullptr;
 }
@@ -94,7 +108,7 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
                                           (long long)B, (long long)G);
   if (B == 0 || M == 0 || O == 0) return 0;
   if (B > 0x7fffffffll || M > 0x7fffffffll || N > 0x7fffffffll) return fail("aitamd_bmm_softmax_bmm_permute: dimension too large");
-  if (K > 128 || O > 128) return fail("aitamd_bmm_softmax_bmm_permute: head dims above 128 are not supported (K=%lld O=%lld)",
+  if (K > 160 || O > 160) return fail("aitamd_bmm_softmax_bmm_permute: head dims above 160 are not supported (K=%lld O=%lld)",
                                       (long long)K, (long long)O);
   if (!out || (N > 0 && (!q || !k || !v))) return fail("aitamd_bmm_softmax_bmm_permute: null pointer");
   AttnParams p{};

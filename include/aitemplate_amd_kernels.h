@@ -190,7 +190,7 @@ AITAMD_API int aitamd_bmm_rcr_permute(int dtype, int algo, const void* a, const 
  * Q [B,M,K], K [B,N,K], V [B,N,O] contiguous; out [B/G, M, G, O] (the "0213"
  * permute of [B/G, G, M, O]); G = number of heads, B % G == 0.  `scale` is
  * rounded to the element type first, as the reference does; causal != 0 masks
- * keys n > m.  K and O up to 128; head dims that are not MFMA multiples are
+ * keys n > m.  K and O up to 160; head dims that are not MFMA multiples are
  * padded on chip only.  Rows whose keys are all masked (N == 0) produce 0.
  * Replaces the generated bmm_softmax_bmm_permute op function's CK call
  * (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:84-110,

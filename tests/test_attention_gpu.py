@@ -72,6 +72,16 @@ def test_every_variant_of_the_small_head_dims(monkeypatch, mode, B, M, N, K, O, 
     _check(B, M, N, K, O, G, causal=causal, scale=scale, seed=mode + N)
 
 
+@pytest.mark.parametrize("B,M,N,K,O,G,causal", [
+    (16, 256, 256, 160, 160, 8, False),     # the deepest attention of Stable Diffusion v1: 1280 channels, 8 heads
+    (8, 100, 77, 160, 160, 8, False),       # its cross-attention over 77 text tokens
+    (4, 130, 200, 136, 160, 2, True),
+    (4, 64, 300, 160, 40, 4, False),
+])
+def test_head_dim_160(B, M, N, K, O, G, causal):
+    _check(B, M, N, K, O, G, causal, seed=11)
+
+
 def test_bf16():
     _check(8, 200, 136, 64, 64, 4, dtype=torch.bfloat16, tol=4e-2)
     _check(8, 100, 100, 40, 40, 8, causal=True, dtype=torch.bfloat16, tol=4e-2)

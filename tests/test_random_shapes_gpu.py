@@ -82,8 +82,8 @@ def test_attention_random_shapes(monkeypatch):
         B = G * rng.choice([1, 2, 3, 8])
         M = rng.choice([1, 7, 31, 32, 33, 100, 128, 129, 255, 256, 257, 300, 511, 700])
         N = rng.choice([1, 5, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 200, 256, 300, 383, 384, 500, 777, 1024])
-        K = rng.choice([8, 16, 24, 32, 40, 48, 64, 72, 96, 128])
-        O = rng.choice([8, 16, 32, 40, 64, 96, 128])
+        K = rng.choice([8, 16, 24, 32, 40, 48, 64, 72, 96, 128, 160])
+        O = rng.choice([8, 16, 32, 40, 64, 96, 128, 160])
         causal = rng.random() < 0.4
         dtype = torch.float16 if rng.random() < 0.7 else torch.bfloat16
         scale = rng.choice([K ** -0.5, K ** -0.5, 0.3, -0.2, 1.0 / 8])
