@@ -151,6 +151,7 @@ def test_bmm_rcr_broadcast_2d_operand():
     ([24], [1020], 1020, 64, 128, 12, False, True),
     ([16], [4096], 64, 40, 40, 8, False, False),
     ([12], [64], 64, 64, 64, 12, True, True),
+    ([16], [256], 77, 160, 160, 8, False, False),   # Stable Diffusion v1: 1280 channels over 8 heads, 77 text tokens
 ])
 def test_bmm_softmax_bmm_permute(bs, ms, N, K, D, heads, causal, copy_op):   # test_bmm_softmax_bmm.py:174-205
     batch_dim = shape_utils.gen_int_var_min_max(bs, name="batch_size")
