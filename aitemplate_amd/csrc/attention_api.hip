@@ -139,10 +139,14 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
   const bool wide = dma && (16 * ks + 32 * ot) <= 112 && ((M + 255) / 256) * B >= 256;
   // two wave groups pay when a CU holds one workgroup anyway: measured 4.5 % faster with 256 workgroups
   // (16 heads x 4096 rows, head dim 40), 2 % slower with 512
-  int mode = wide ? (((M + 255) / 256) * B <= 256 ? 2 : 1) : 0;
+  // (wave groups take alternate key tiles: with fewer than four tiles there is nothing to share out - the 77 text
+  // tokens of a cross-attention are a single tile)
+  const int64_t bn = (16 * ks + 32 * ot) <= 112 ? 128 : 64;
+  const bool groups_pay = N >= 4 * bn;
+  int mode = wide ? ((((M + 255) / 256) * B <= 256 && groups_pay) ? 2 : 1) : 0;
   // grids of 128-row workgroups that leave CUs idle take the two-group form of those too: 8-19 % faster from 48 to
   // 256 workgroups (head dims 40 and 64), 7 % slower at 384
-  if (mode == 0 && dma && ((M + 127) / 128) * B <= 256) mode = 3;
+  if (mode == 0 && dma && groups_pay && ((M + 127) / 128) * B <= 256) mode = 3;
   // AITAMD_ATTN_MODE=0|1|2|3 forces a variant where the shape allows it (a test and measurement knob)
   if (const char* forced = getenv("AITAMD_ATTN_MODE")) {
     const int m = atoi(forced);
