@@ -1,0 +1,74 @@
+"""mem_eff_attention: fused multi-head attention on [batch, heads, seq, head_dim] operands,
+softmax(Q K^T / sqrt(head_dim)) V, written as [batch, seq, heads, head_dim_v].
+
+Counterpart of python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-263 (constructor arguments,
+`__call__(q, k, v, lengths_kv=None, lengths_q=None)`, output shape, exec keys, `_get_op_attributes`).  The
+reference's ROCm hook (backend/rocm/attention/mem_eff_attention.py) only has a grouped variable-length form that
+reads the device-side lengths on the host and is skipped by its own test on ROCm (tests/unittest/ops/
+test_attention.py:705); the fixed-length form built here is the one `nn.CrossAttention` uses
+(frontend/nn/attention.py:338) with the meaning its CUDA backend gives it.  Variable sequence lengths raise."""
+import itertools
+from collections import OrderedDict
+from typing import Optional
+
+from ....backend import registry
+from ....backend.target import Target
+from ...base import Operator, Tensor
+
+
+class mem_eff_attention(Operator):
+    def __init__(self, causal, dropout=0, variable_seq_length_kv=False, variable_seq_length_q=False,
+                 use_grouped_fmha=False) -> None:
+        super().__init__()
+        assert dropout == 0
+        if variable_seq_length_kv or variable_seq_length_q:
+            raise NotImplementedError("mem_eff_attention with variable sequence lengths is not built for gfx950")
+        self._attrs["op"] = "mem_eff_attention"
+        self._attrs["has_profiler"] = False
+        self._attrs["dropout"] = dropout
+        self._attrs["causal"] = causal
+        self._attrs["variable_seq_length_kv"] = variable_seq_length_kv
+        self._attrs["variable_seq_length_q"] = variable_seq_length_q
+        self._attrs["head_size"] = -1
+        self._attrs["workspace"] = 0
+        self._attrs["use_grouped_fmha"] = use_grouped_fmha
+
+    def _infer_shapes(self, q: Tensor, v: Tensor):
+        qs, vs = q._attrs["shape"], v._attrs["shape"]
+        # [batch, heads, seq, head_dim] -> [batch, seq, heads, head_dim_v]
+        return [qs[0], qs[2], qs[1], vs[-1]]
+
+    def __call__(self, q: Tensor, k: Tensor, v: Tensor, lengths_kv: Optional[Tensor] = None,
+                 lengths_q: Optional[Tensor] = None) -> Tensor:
+        if lengths_kv is not None or lengths_q is not None:
+            raise NotImplementedError("mem_eff_attention with variable sequence lengths is not built for gfx950")
+        for t, name in ((q, "q"), (k, "k"), (v, "v")):
+            if len(t._attrs["shape"]) != 4:
+                raise RuntimeError(f"mem_eff_attention: {name} must be [batch, heads, seq, head_dim]")
+        for dim in (1, 3):
+            if len(q._attrs["shape"][dim]._attrs["values"]) != 1:
+                raise RuntimeError("mem_eff_attention: the number of heads and the head dim must be static")
+        if q._attrs["shape"][3] != k._attrs["shape"][3] or k._attrs["shape"][2] != v._attrs["shape"][2]:
+            raise RuntimeError("mem_eff_attention: q / k head dims and k / v sequence lengths must agree")
+        self._attrs["head_size"] = v._attrs["shape"][3]._attrs["values"][0]
+        self._attrs["inputs"] = [q, k, v]
+        self._set_depth()
+        self._extract_exec_path(q)
+        output = Tensor(self._infer_shapes(q, v), src_ops={self}, dtype=q._attrs["dtype"])
+        self._attrs["outputs"] = [output]
+        return output
+
+    def _get_op_attributes(self):
+        return {"causal": self._attrs["causal"]}
+
+    def _gen_exec_key(self, shape):
+        return (f"batch_size == {shape[0]} && num_heads == {shape[1]} && seq_len == {shape[2]} && "
+                f"head_sizes == {shape[3]}")
+
+    def _extract_exec_path(self, x: Tensor):
+        values = [dim._attrs["values"] for dim in x._attrs["shape"]]
+        self._attrs["exec_path"] = OrderedDict((self._gen_exec_key(s), "") for s in itertools.product(*values))
+
+    def gen_function(self) -> str:
+        target = Target.current()
+        return registry.get(f"{target.name()}.{self._attrs['op']}.gen_function")(self._attrs)

@@ -11,9 +11,14 @@ Counterpart of the ROCm branch of python/aitemplate/frontend/nn/attention.py:95-
            -> [B, S, dim]
 
 Three kernels per block: two GEMMs and one attention launch; the split and every reshape are views.
-The CUDA-only pieces of the reference module (flash attention on a packed tensor, cu_length, the
-memory-efficient kernel) have no counterpart here; `mask_seq` needs dynamic_slice / concatenate, which
-this backend does not have."""
+The CUDA-only pieces of the reference module (flash attention on a packed tensor, cu_length) have no
+counterpart here; `mask_seq` needs dynamic_slice / concatenate, which this backend does not have.
+
+nn.CrossAttention (python/aitemplate/frontend/nn/attention.py:289-400): separate Q / K / V projections of three
+inputs, mem_eff_attention on [B, heads, S, head_dim] operands, output projection.  The reference permutes the
+projected tensors with a stand-alone permute op; here each projection writes the permuted layout itself
+(Linear specialization="permute", shape=(seq, 1, heads), layout="m2n3": [B*S, dim] -> [1, B, heads, S, head_dim]),
+so the block is four GEMMs and one attention launch."""
 from ...compiler import ops
 from .dropout import Dropout
 from .linear import Linear
@@ -34,7 +39,7 @@ class MultiheadAttention(Module):
         if mask_seq:
             raise NotImplementedError("mask_seq needs dynamic_slice and concatenate, which this backend lacks")
         if use_mem_eff:
-            raise NotImplementedError("mem_eff_attention is a CUDA kernel of the reference; ROCm uses "
+            raise NotImplementedError("use_mem_eff is the CUDA branch of the reference module; ROCm uses "
                                       "bmm_softmax_bmm_permute")
         self.num_heads = num_heads
         self.scale = (dim // num_heads) ** -0.5
@@ -74,3 +79,55 @@ class MultiheadAttention(Module):
             x = self.proj(attn_output)
         x = self.proj_drop(x)
         return ops.reshape()(x, [batch, seq, hidden])
+
+
+class CrossAttention(Module):
+    r"""Cross Multi-head Attention: queries from one sequence, keys and values from another.
+
+    Args mirror the reference: dim, seq_len, seq_len_kv, num_heads, qkv_bias=False, attn_drop=0.0, proj_drop=0.0,
+    has_residual=True, causal=False, dtype="float16".  forward(q, k, v[, residual]) with q: [B, seq_len, dim] and
+    k, v: [B, seq_len_kv, dim]; returns [B, seq_len, dim]."""
+
+    def __init__(self, dim, seq_len, seq_len_kv, num_heads, qkv_bias=False, attn_drop=0.0, proj_drop=0.0,
+                 has_residual=True, causal=False, dtype="float16"):
+        super().__init__()
+        assert dim % num_heads == 0, f"dim {dim} should be divisible by num_heads {num_heads}"
+        self.num_heads = num_heads
+        self.causal = causal
+        self.has_residual = has_residual
+        self.dim = dim
+        self.op = ops.mem_eff_attention(causal=causal)
+
+        def permuting(seq):
+            return Linear(dim, dim, bias=qkv_bias, specialization="permute", shape=(seq, 1, num_heads), layout="m2n3",
+                          dtype=dtype)
+
+        self.proj_q = permuting(seq_len)
+        self.proj_k = permuting(seq_len_kv)
+        self.proj_v = permuting(seq_len_kv)
+        self.attn_drop = Dropout(attn_drop, dtype=dtype)
+        self.proj = Linear(dim, dim, specialization="add" if has_residual else None, dtype=dtype)
+        self.proj_drop = Dropout(proj_drop, dtype=dtype)
+
+    def attention(self, q, k, v):
+        """[B, S, dim] inputs -> [B, S, heads, head_dim]"""
+        head_dim = self.dim // self.num_heads
+
+        def heads_first(proj, x):
+            batch, seq, _ = [d.value() for d in x._attrs["shape"]]
+            return ops.reshape()(proj(x), [batch, self.num_heads, seq, head_dim])  # [1, B, H, S, D] viewed as 4-D
+
+        return self.op(heads_first(self.proj_q, q), heads_first(self.proj_k, k), heads_first(self.proj_v, v))
+
+    def forward(self, *args):
+        assert len(args) >= 3
+        x = args[0]
+        batch, seq, _ = [d.value() for d in x._attrs["shape"]]
+        attn_output = ops.reshape()(self.attention(args[0], args[1], args[2]), [batch * seq, self.dim])
+        if self.has_residual:
+            assert len(args) == 4
+            x = self.proj(attn_output, args[3])
+        else:
+            x = self.proj(attn_output)
+        x = self.proj_drop(x)
+        return ops.reshape()(x, [batch, seq, self.dim])

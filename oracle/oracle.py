@@ -171,6 +171,28 @@ def torch_multihead_attention(x, qkv_w, qkv_b, proj_w, proj_b, residual, num_hea
     return y.reshape(B, S, D)
 
 
+def torch_cross_attention(q_in, k_in, v_in, wq, wk, wv, bq, bk, bv, proj_w, proj_b, residual, num_heads: int,
+                          causal: bool = False) -> torch.Tensor:
+    """fp32 cross-attention block (python/aitemplate/frontend/nn/attention.py:289-400): separate q, k and v
+    projections, softmax(q k^T / sqrt(d)) v per head, output projection (+ residual).
+    q_in: [B, S, D]; k_in, v_in: [B, Skv, D]."""
+    B, S, D = q_in.shape
+    Skv = k_in.shape[1]
+    d = D // num_heads
+    lin = torch.nn.functional.linear
+    q = lin(_f(q_in), _f(wq), _f(bq)).reshape(B, S, num_heads, d).permute(0, 2, 1, 3)
+    k = lin(_f(k_in), _f(wk), _f(bk)).reshape(B, Skv, num_heads, d).permute(0, 2, 1, 3)
+    v = lin(_f(v_in), _f(wv), _f(bv)).reshape(B, Skv, num_heads, d).permute(0, 2, 1, 3)
+    s = torch.matmul(q, k.transpose(-1, -2)) * (d ** -0.5)
+    if causal:
+        s = s.masked_fill(torch.triu(torch.ones(S, Skv, dtype=torch.bool), diagonal=1), float("-inf"))
+    o = torch.matmul(torch.softmax(s, dim=-1), v).permute(0, 2, 1, 3).reshape(B * S, D)
+    y = lin(o, _f(proj_w), _f(proj_b))
+    if residual is not None:
+        y = y + _f(residual).reshape(B * S, D)
+    return y.reshape(B, S, D)
+
+
 def torch_bmm_rcr(q, k) -> torch.Tensor:
     q, k = _f(q), _f(k)
     if q.dim() == 2:

@@ -173,6 +173,41 @@ def test_bmm_softmax_bmm_permute(bs, ms, N, K, D, heads, causal, copy_op):   # t
         torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("B,H,M,N,D,Dv,causal,copy_op", [
+    (2, 8, 256, 256, 40, 40, False, False),     # self-attention of a Stable Diffusion block
+    (2, 8, 200, 77, 40, 40, False, True),       # nn.CrossAttention over 77 text tokens (frontend/nn/attention.py:338)
+    (3, 4, 100, 100, 64, 64, True, False),
+    (1, 8, 64, 130, 160, 160, False, False),
+])
+def test_mem_eff_attention_fixed_lengths(B, H, M, N, D, Dv, causal, copy_op):
+    # the reference checks this op against softmax(q k^T / sqrt(d)) v, transposed to [batch, seq, heads, d]
+    # (tests/unittest/ops/test_attention.py:456-700; skipped there on ROCm)
+    print(f"case compile_model mem_eff_attention B={B} H={H} M={M} N={N} D={D} causal={causal}", flush=True)
+    Q = Tensor(shape=[B, H, M, D], dtype="float16", name="q", is_input=True)
+    K = Tensor(shape=[B, H, N, D], dtype="float16", name="k", is_input=True)
+    V = Tensor(shape=[B, H, N, Dv], dtype="float16", name="v", is_input=True)
+    OP = ops.mem_eff_attention(causal=causal)
+    if copy_op:
+        OP = ops.mem_eff_attention(**OP._get_op_attributes())
+    Y = _mark_output(OP(Q, K, V))
+    module = compile_model(Y, detect_target(), WORKDIR, f"mem_eff_attention_{next(_counter)}")
+    q, k, v = _rand((B, H, M, D), 1), _rand((B, H, N, D), 2), _rand((B, H, N, Dv), 3)
+    y = torch.empty(B, M, H, Dv, dtype=torch.float16, device="cuda")
+    out = module.run_with_tensors({"q": q.cuda(), "k": k.cuda(), "v": v.cuda()}, [y])
+    assert tuple(out["output_0"].shape) == (B, M, H, Dv)
+    p = torch.matmul(q.float(), k.float().transpose(-1, -2)) * D ** -0.5
+    if causal:
+        p = p.masked_fill(torch.ones(M, N, dtype=torch.bool).triu(1), float("-inf"))
+    want = torch.matmul(torch.softmax(p, dim=-1), v.float()).permute(0, 2, 1, 3).half().float()
+    torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
+    module.close()
+
+
+def test_mem_eff_attention_variable_lengths_are_refused():
+    with pytest.raises(NotImplementedError):
+        ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)
+
+
 @pytest.mark.parametrize("B,M,N,K,D,copy_op", [(24, 256, 256, 64, 64, False), (5, 100, 49, 40, 40, True)])
 def test_bmm_softmax_bmm(B, M, N, K, D, copy_op):   # the non-permuted op (reference: test_bmm_softmax_bmm.py:59-118)
     X = Tensor(shape=[B, M, K], name="input_0", is_input=True)
@@ -311,6 +346,53 @@ def test_nn_multihead_attention(B, S, D, H, qkv_bias, residual, causal):
     feed = {"input_0": x.cuda()}
     if residual:
         feed["input_1"] = res.cuda()
+    y = torch.empty(B, S, D, dtype=torch.float16, device="cuda")
+    module.run_with_tensors(feed, [y])
+    torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)
+    module.close()
+
+
+@pytest.mark.parametrize("B,S,Skv,D,H,qkv_bias,residual,causal", [
+    (2, 1024, 77, 320, 8, False, True, False),   # the image-to-text attention of a diffusion UNet block
+    (2, 64, 200, 512, 8, True, False, False),
+    (3, 96, 96, 256, 4, False, True, True),
+    (1, 50, 33, 96, 4, True, True, False),
+])
+def test_nn_cross_attention(B, S, Skv, D, H, qkv_bias, residual, causal):
+    """frontend.nn.CrossAttention (three projections stored head-major, mem_eff_attention on the fused
+    kernel, projection with the residual add) against the fp32 PyTorch block.  Tolerance 2e-2 as for the
+    self-attention block."""
+    from aitemplate_amd.frontend import nn
+
+    print(f"case compile_model CrossAttention B={B} S={S} Skv={Skv} D={D} H={H} bias={qkv_bias} "
+          f"res={residual} causal={causal}", flush=True)
+    att = nn.CrossAttention(D, S, Skv, H, qkv_bias=qkv_bias, has_residual=residual, causal=causal)
+    att.name_parameter_tensor()
+    Q = Tensor(shape=[B, S, D], dtype="float16", name="input_q", is_input=True)
+    K = Tensor(shape=[B, Skv, D], dtype="float16", name="input_k", is_input=True)
+    V = Tensor(shape=[B, Skv, D], dtype="float16", name="input_v", is_input=True)
+    args = [Q, K, V]
+    if residual:
+        args.append(Tensor(shape=[B * S, D], dtype="float16", name="input_r", is_input=True))
+    Y = _mark_output(att(*args))
+    module = compile_model(Y, detect_target(), WORKDIR, f"cross_attention_{next(_counter)}")
+    q, k, v = _rand((B, S, D), 1), _rand((B, Skv, D), 2), _rand((B, Skv, D), 3)
+    res = _rand((B * S, D), 4)
+    w = {n: _rand((D, D), 5 + i, D ** -0.5) for i, n in enumerate(("proj_q", "proj_k", "proj_v", "proj"))}
+    b = {n: _rand((D,), 9 + i, 0.5) for i, n in enumerate(("proj_q", "proj_k", "proj_v", "proj"))}
+    consts = {f"{n}_weight": t.cuda() for n, t in w.items()}
+    consts["proj_bias"] = b["proj"].cuda()
+    if qkv_bias:
+        consts.update({f"{n}_bias": b[n].cuda() for n in ("proj_q", "proj_k", "proj_v")})
+    assert sorted(module.get_constant_names()) == sorted(consts)
+    module.set_many_constants_with_tensors(consts)
+    bias = (lambda n: b[n]) if qkv_bias else (lambda n: None)
+    want = oracle.torch_cross_attention(q, k, v, w["proj_q"], w["proj_k"], w["proj_v"], bias("proj_q"),
+                                        bias("proj_k"), bias("proj_v"), w["proj"], b["proj"],
+                                        res if residual else None, H, causal)
+    feed = {"input_q": q.cuda(), "input_k": k.cuda(), "input_v": v.cuda()}
+    if residual:
+        feed["input_r"] = res.cuda()
     y = torch.empty(B, S, D, dtype=torch.float16, device="cuda")
     module.run_with_tensors(feed, [y])
     torch.testing.assert_close(y.cpu().float(), want, atol=2e-2, rtol=2e-2)

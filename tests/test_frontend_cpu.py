@@ -581,6 +581,78 @@ def test_multihead_attention_block_compiles_to_three_kernels(tmp_path, monkeypat
         nn.MultiheadAttention(D, B, S, H, mask_seq=4)
 
 
+def test_mem_eff_attention_op_shapes_keys_and_hooks():
+    """Operator attributes, output shape and exec keys as python/aitemplate/compiler/ops/attention/
+    mem_eff_attention.py:49-263 gives them; variable sequence lengths are refused, not approximated."""
+    import aitemplate_amd.backend.rocm  # noqa: F401  registers the hooks
+
+    q = Tensor([2, 8, 64, 40], name="q", is_input=True)
+    k = Tensor([2, 8, 77, 40], name="k", is_input=True)
+    v = Tensor([2, 8, 77, 48], name="v", is_input=True)
+    op = ops.mem_eff_attention(causal=False)
+    y = op(q, k, v)
+    assert [d.value() for d in y.shape()] == [2, 64, 8, 48]
+    assert op._get_op_attributes() == {"causal": False}
+    assert op._attrs["head_size"] == 48 and op._attrs["workspace"] == 0
+    assert list(op._attrs["exec_path"]) == ["batch_size == 2 && num_heads == 8 && seq_len == 64 && head_sizes == 40"]
+    op._attrs["name"] = "mem_eff_attention_0"
+    for t in (q, k, v):
+        for i, d in enumerate(t._attrs["shape"]):
+            d._attrs["name"] = f"{t._attrs['name']}_dim_{i}"
+    y._attrs["name"] = "y"
+    decl = registry.get("rocm.mem_eff_attention.func_decl")(op._attrs)
+    assert decl.startswith("void mem_eff_attention_0(void* output, const void* q, const void* k, const void* v, "
+                           "int64_t* batch_size, int64_t* seq_len, int64_t* seq_len_kv, int num_heads, ")
+    call = registry.get("rocm.mem_eff_attention.func_call")(op._attrs)
+    assert call == f"  mem_eff_attention_0(y, q, k, v, &q_dim_0, &q_dim_2, &k_dim_2, 8, 40, 48, {40 ** -0.5!r}f, stream);"
+    causal_op = ops.mem_eff_attention(causal=True)
+    causal_op(q, k, v)
+    causal_op._attrs["name"] = "mem_eff_attention_1"
+    with detect_target():
+        src = op.gen_function()
+        causal_src = causal_op.gen_function()
+    assert "aitamd_bmm_softmax_bmm_permute(0, q, k, v, output, B, *seq_len, *seq_len_kv, head_dim, head_dim_v," in src
+    assert "num_heads, softmax_scale, 0, stream)" in src
+    assert "num_heads, softmax_scale, 1, stream)" in causal_src
+    with pytest.raises(NotImplementedError):
+        ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)
+    with pytest.raises(NotImplementedError):
+        ops.mem_eff_attention(causal=False)(q, k, v, lengths_kv=Tensor([2], name="len", dtype="int32", is_input=True))
+    with pytest.raises(RuntimeError, match="head dims"):
+        ops.mem_eff_attention(causal=False)(q, Tensor([2, 8, 77, 32], name="k2", is_input=True), v)
+
+
+def test_cross_attention_block_compiles_to_five_kernels(tmp_path, monkeypatch):
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    reset_name_counters()
+    B, S, Skv, D, H = 2, 64, 77, 128, 4
+    q = Tensor([B, S, D], name="q", is_input=True)
+    k = Tensor([B, Skv, D], name="k", is_input=True)
+    v = Tensor([B, Skv, D], name="v", is_input=True)
+    res = Tensor([B * S, D], name="res", is_input=True)
+    att = nn.CrossAttention(D, S, Skv, H)
+    att.name_parameter_tensor()
+    assert [n for n, _ in att.named_parameters()] == ["proj_q.weight", "proj_k.weight", "proj_v.weight",
+                                                      "proj.weight", "proj.bias"]
+    y = att(q, k, v, res)
+    y._attrs["is_output"] = True
+    y._attrs["name"] = "y"
+    assert [d.value() for d in y.shape()] == [B, S, D]
+    import torch
+
+    if torch.cuda.is_available():
+        compile_model(y, detect_target(), str(tmp_path), "cross").close()
+    else:
+        with pytest.raises(RuntimeError, match="AITemplateModelContainerCreate"):
+            compile_model(y, detect_target(), str(tmp_path), "cross")
+    model_src = (tmp_path / "cross" / "model-generated.cpp").read_text()
+    entries = [e.rsplit("_", 1)[0] for e in re.findall(r'OpEntry\{"(\w+)"', model_src)]
+    assert sorted(entries) == sorted(["gemm_rcr_permute_m2n3"] * 3 + ["mem_eff_attention", "gemm_rcr_bias_add"]), entries
+    assert entries[-2:] == ["mem_eff_attention", "gemm_rcr_bias_add"]
+    assert f", {S}, 1, {H}, stream);" in model_src and f", {Skv}, 1, {H}, stream);" in model_src
+    assert f", {H}, {D // H}, {D // H}, {(D // H) ** -0.5!r}f, stream);" in model_src
+
+
 # ---- fuse_mm_elementwise ----------------------------------------------------------------------
 def _fuse(outputs):
     outputs = list(outputs)
