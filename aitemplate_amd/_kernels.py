@@ -83,6 +83,7 @@ EXPORTED_SYMBOLS = [
     "aitamd_gemm_heuristic_algo_layout",
     "aitamd_bmm_rcr",
     "aitamd_bmm_softmax_bmm_permute",
+    "aitamd_mem_eff_attention",
 ]
 
 _lock = threading.Lock()
@@ -141,6 +142,9 @@ def load() -> ctypes.CDLL:
         lib.aitamd_bmm_softmax_bmm_permute.restype = i32
         lib.aitamd_bmm_softmax_bmm_permute.argtypes = [i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64,
                                                        ctypes.c_float, i32, vp]
+        lib.aitamd_mem_eff_attention.restype = i32
+        lib.aitamd_mem_eff_attention.argtypes = [i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, i32,
+                                                 vp, vp]
         _lib = lib
         return lib
 

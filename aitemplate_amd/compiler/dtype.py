@@ -1,6 +1,7 @@
 """dtype vocabulary of the IR (counterpart of python/aitemplate/compiler/dtype.py)."""
 
-_ALIASES = {"half": "float16", "fp16": "float16", "bf16": "bfloat16", "float": "float32", "fp32": "float32"}
+_ALIASES = {"half": "float16", "fp16": "float16", "bf16": "bfloat16", "float": "float32", "fp32": "float32",
+            "int": "int32"}
 _SIZES = {"float16": 2, "bfloat16": 2, "float32": 4, "int32": 4, "int64": 8, "bool": 1}
 # AITemplateDtype enum values of the C ABI (static/include/model_interface.h)
 _ENUM = {"float16": 1, "float32": 2, "int32": 3, "int64": 4, "bool": 5, "bfloat16": 6}

@@ -3,10 +3,12 @@ softmax(Q K^T / sqrt(head_dim)) V, written as [batch, seq, heads, head_dim_v].
 
 Counterpart of python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-263 (constructor arguments,
 `__call__(q, k, v, lengths_kv=None, lengths_q=None)`, output shape, exec keys, `_get_op_attributes`).  The
-reference's ROCm hook (backend/rocm/attention/mem_eff_attention.py) only has a grouped variable-length form that
-reads the device-side lengths on the host and is skipped by its own test on ROCm (tests/unittest/ops/
-test_attention.py:705); the fixed-length form built here is the one `nn.CrossAttention` uses
-(frontend/nn/attention.py:338) with the meaning its CUDA backend gives it.  Variable sequence lengths raise."""
+reference's ROCm hook (backend/rocm/attention/mem_eff_attention.py) reads the device-side lengths on the host and is
+skipped by its own test on ROCm (tests/unittest/ops/test_attention.py:705); the meaning built here is the one that
+test states for every backend (test_attention.py:504-523, 593, 661-664): `lengths_kv` [batch, 1] int32 is a key-padding
+mask (batch entry b attends to its first lengths_kv[b] keys), rows past `lengths_q` are unspecified, so `lengths_q` is
+accepted and not read.  `nn.CrossAttention` uses the fixed-length form (frontend/nn/attention.py:338).
+`use_grouped_fmha` selects between two CUDA kernels in the reference and changes nothing here."""
 import itertools
 from collections import OrderedDict
 from typing import Optional
@@ -21,8 +23,6 @@ class mem_eff_attention(Operator):
                  use_grouped_fmha=False) -> None:
         super().__init__()
         assert dropout == 0
-        if variable_seq_length_kv or variable_seq_length_q:
-            raise NotImplementedError("mem_eff_attention with variable sequence lengths is not built for gfx950")
         self._attrs["op"] = "mem_eff_attention"
         self._attrs["has_profiler"] = False
         self._attrs["dropout"] = dropout
@@ -40,8 +40,6 @@ class mem_eff_attention(Operator):
 
     def __call__(self, q: Tensor, k: Tensor, v: Tensor, lengths_kv: Optional[Tensor] = None,
                  lengths_q: Optional[Tensor] = None) -> Tensor:
-        if lengths_kv is not None or lengths_q is not None:
-            raise NotImplementedError("mem_eff_attention with variable sequence lengths is not built for gfx950")
         for t, name in ((q, "q"), (k, "k"), (v, "v")):
             if len(t._attrs["shape"]) != 4:
                 raise RuntimeError(f"mem_eff_attention: {name} must be [batch, heads, seq, head_dim]")
@@ -52,6 +50,13 @@ class mem_eff_attention(Operator):
             raise RuntimeError("mem_eff_attention: q / k head dims and k / v sequence lengths must agree")
         self._attrs["head_size"] = v._attrs["shape"][3]._attrs["values"][0]
         self._attrs["inputs"] = [q, k, v]
+        for flag, lengths, name in ((self._attrs["variable_seq_length_kv"], lengths_kv, "lengths_kv"),
+                                    (self._attrs["variable_seq_length_q"], lengths_q, "lengths_q")):
+            if flag:
+                assert lengths is not None, f"mem_eff_attention: {name} is required"
+                if lengths._attrs["dtype"] != "int32":
+                    raise RuntimeError(f"mem_eff_attention: {name} must be int32, got {lengths._attrs['dtype']}")
+                self._attrs["inputs"].append(lengths)
         self._set_depth()
         self._extract_exec_path(q)
         output = Tensor(self._infer_shapes(q, v), src_ops={self}, dtype=q._attrs["dtype"])
@@ -59,7 +64,9 @@ class mem_eff_attention(Operator):
         return output
 
     def _get_op_attributes(self):
-        return {"causal": self._attrs["causal"]}
+        # (the reference returns "causal" only, so a copy of a variable-length op loses its flags there)
+        return {name: self._attrs[name] for name in ("causal", "variable_seq_length_kv", "variable_seq_length_q",
+                                                     "use_grouped_fmha")}
 
     def _gen_exec_key(self, shape):
         return (f"batch_size == {shape[0]} && num_heads == {shape[1]} && seq_len == {shape[2]} && "

@@ -99,18 +99,20 @@ float round_to_elem(float x, int dtype) {
 
 using namespace aitamd;
 
-extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const void* k, const void* v, void* out,
-                                              int64_t B, int64_t M, int64_t N, int64_t K, int64_t O, int64_t G,
-                                              float scale, int causal, void* stream) {
-  if (dtype != 0 && dtype != 1) return fail("aitamd_bmm_softmax_bmm_permute: bad dtype %d", dtype);
-  if (B < 0 || M < 0 || N < 0 || K < 0 || O < 0) return fail("aitamd_bmm_softmax_bmm_permute: negative dimension");
-  if (G <= 0 || (B % G) != 0) return fail("aitamd_bmm_softmax_bmm_permute: batch %lld is not a multiple of heads %lld",
+namespace {
+
+int attention_entry(const char* who, int dtype, const void* q, const void* k, const void* v, void* out, int64_t B,
+                    int64_t M, int64_t N, int64_t K, int64_t O, int64_t G, float scale, int causal,
+                    const int32_t* kv_len, void* stream) {
+  if (dtype != 0 && dtype != 1) return fail("%s: bad dtype %d", who, dtype);
+  if (B < 0 || M < 0 || N < 0 || K < 0 || O < 0) return fail("%s: negative dimension", who);
+  if (G <= 0 || (B % G) != 0) return fail("%s: batch %lld is not a multiple of heads %lld", who,
                                           (long long)B, (long long)G);
   if (B == 0 || M == 0 || O == 0) return 0;
-  if (B > 0x7fffffffll || M > 0x7fffffffll || N > 0x7fffffffll) return fail("aitamd_bmm_softmax_bmm_permute: dimension too large");
-  if (K > 160 || O > 160) return fail("aitamd_bmm_softmax_bmm_permute: head dims above 160 are not supported (K=%lld O=%lld)",
+  if (B > 0x7fffffffll || M > 0x7fffffffll || N > 0x7fffffffll) return fail("%s: dimension too large", who);
+  if (K > 160 || O > 160) return fail("%s: head dims above 160 are not supported (K=%lld O=%lld)", who,
                                       (long long)K, (long long)O);
-  if (!out || (N > 0 && (!q || !k || !v))) return fail("aitamd_bmm_softmax_bmm_permute: null pointer");
+  if (!out || (N > 0 && (!q || !k || !v))) return fail("%s: null pointer", who);
   AttnParams p{};
   p.q = q;
   p.k = k;
@@ -126,6 +128,7 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
   // (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:47-51)
   p.scale_log2e = round_to_elem(scale, dtype) * 1.4426950408889634f;
   p.causal = causal ? 1 : 0;
+  p.kv_len = kv_len;
   const int ks = (int)((K + 15) / 16) > 0 ? (int)((K + 15) / 16) : 1;
   const int ot = (int)((O + 31) / 32);
   const bool vec = (K % 8 == 0) && (O % 8 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15) == 0) &&
@@ -166,8 +169,28 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
                    : (mode == 1 ? pick<bf16, true, true, 1>(ks, ot)
                                 : (dma ? pick<bf16, true, true, 0>(ks, ot)
                                        : (vec ? pick<bf16, true, false, 0>(ks, ot) : pick<bf16, false, false, 0>(ks, ot))));
-  if (!fn) return fail("aitamd_bmm_softmax_bmm_permute: no instance for K=%lld O=%lld", (long long)K, (long long)O);
+  if (!fn) return fail("%s: no instance for K=%lld O=%lld", who, (long long)K, (long long)O);
   const hipError_t e = fn(p, reinterpret_cast<hipStream_t>(stream));
-  if (e != hipSuccess) return fail("aitamd_bmm_softmax_bmm_permute: launch failed: %s", hipGetErrorString(e));
+  if (e != hipSuccess) return fail("%s: launch failed: %s", who, hipGetErrorString(e));
   return 0;
+}
+
+}  // namespace
+
+extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const void* k, const void* v, void* out,
+                                              int64_t B, int64_t M, int64_t N, int64_t K, int64_t O, int64_t G,
+                                              float scale, int causal, void* stream) {
+  return attention_entry("aitamd_bmm_softmax_bmm_permute", dtype, q, k, v, out, B, M, N, K, O, G, scale, causal, nullptr,
+                         stream);
+}
+
+extern "C" int aitamd_mem_eff_attention(int dtype, const void* q, const void* k, const void* v, void* out,
+                                        int64_t batch, int64_t heads, int64_t seq_q, int64_t seq_kv, int64_t head_dim,
+                                        int64_t head_dim_v, float scale, int causal, const int32_t* lengths_kv,
+                                        void* stream) {
+  if (batch < 0 || heads <= 0) return fail("aitamd_mem_eff_attention: bad batch %lld or heads %lld", (long long)batch,
+                                           (long long)heads);
+  if (batch > 0x7fffffffll / heads) return fail("aitamd_mem_eff_attention: dimension too large");
+  return attention_entry("aitamd_mem_eff_attention", dtype, q, k, v, out, batch * heads, seq_q, seq_kv, head_dim,
+                         head_dim_v, heads, scale, causal, lengths_kv, stream);
 }

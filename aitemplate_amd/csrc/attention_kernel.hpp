@@ -42,6 +42,9 @@ struct AttnParams {
   int32_t B, M, N, K, O, G;
   float scale_log2e;  // scale (already rounded to the element type) * log2(e)
   int32_t causal;
+  // Optional, device memory, B / G entries: batch entry b only attends to its first kv_len[b / G] keys (clamped to
+  // [0, N]); the later rows of K and V are never read.  Null: all N keys.
+  const int32_t* kv_len;
 };
 
 // NW_ waves (32 query rows each) share the K / V tiles; NS_ LDS stages.  The register-staged
@@ -192,6 +195,12 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     const T* Qb = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.M * p.K;
     const T* Kb = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.N * p.K;
     const T* Vb = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.N * p.O;
+    // keys of this batch entry (uniform over the workgroup)
+    int N = p.N;
+    if (p.kv_len != nullptr) {
+      const int len = __builtin_amdgcn_readfirstlane(p.kv_len[b / p.G]);
+      N = len < 0 ? 0 : (len < N ? len : N);
+    }
 
     // ---- Q fragments (B operand of S^T = K Q^T): lane (q = r32, k = 16 ks + 8 h + j)
     vec8 qf[KS];
@@ -241,13 +250,13 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
       for (int i = 0; i < Tile::K_IT; ++i) {
         const int c = tid + i * Tile::NT;
         const int row = c / (KP / 8), col = (c % (KP / 8)) * 8;
-        kreg[i] = (c < Tile::K_CHUNKS) ? gather(Kb, n0 + row, col, p.N, p.K) : u32x4{0, 0, 0, 0};
+        kreg[i] = (c < Tile::K_CHUNKS) ? gather(Kb, n0 + row, col, N, p.K) : u32x4{0, 0, 0, 0};
       }
 #pragma unroll
       for (int i = 0; i < Tile::V_IT; ++i) {
         const int c = tid + i * Tile::NT;
         const int row = c / (OP / 8), col = (c % (OP / 8)) * 8;
-        vreg[i] = (c < Tile::V_CHUNKS) ? gather(Vb, n0 + row, col, p.N, p.O) : u32x4{0, 0, 0, 0};
+        vreg[i] = (c < Tile::V_CHUNKS) ? gather(Vb, n0 + row, col, N, p.O) : u32x4{0, 0, 0, 0};
       }
     };
     auto store_tiles = [&](int stage) {
@@ -301,13 +310,13 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         const uint32_t off =
             d_off[i] != kOobOffset ? d_off[i] + (uint32_t)(n0 * (is_k ? p.K : p.O) * 2) : kOobOffset;
         T* dst = is_k ? dK + j * 512 : dV + (j - KL) * 512;
-        const __amdgpu_buffer_rsrc_t r = make_rsrc(is_k ? Kb : Vb, (uint32_t)((int64_t)p.N * (is_k ? p.K : p.O) * 2));
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(is_k ? Kb : Vb, (uint32_t)((int64_t)N * (is_k ? p.K : p.O) * 2));
         __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)dst, 16, off, 0, 0, 0);
       }
     };
 
     // keys this workgroup has to visit (causal: nothing right of the last query row)
-    int n_end = p.N;
+    int n_end = N;
     if (p.causal) {
       const int last = m0 + Tile::BM;
       n_end = last < n_end ? last : n_end;
@@ -412,7 +421,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         // p = exp2(s * c - m * c) is one FMA and one v_exp per score (c > 0: a negative scale was moved into
         // the Q fragments).  Only blocks that reach past N or touch the causal diagonal pay for masking; the
         // test is wave-uniform, so it costs one scalar branch per block.
-        const bool need_mask = (nb + 32 * KB > p.N) || (p.causal && nb + 32 * KB - 1 > m0 + wave_u * 32);
+        const bool need_mask = (nb + 32 * KB > N) || (p.causal && nb + 32 * KB - 1 > m0 + wave_u * 32);
         float alpha = 1.0f;
         vec8 pf[2 * KB];  // P^T fragments of the block's 16-key steps
         auto softmax_block = [&](auto masked_tag) {
@@ -424,7 +433,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
 #pragma unroll
               for (int e = 0; e < 16; ++e) {
                 const int n = nb + kb * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                dead[kb][e] = (n >= p.N) || (p.causal && n > q_row);
+                dead[kb][e] = (n >= N) || (p.causal && n > q_row);
               }
           }
           float text = -INFINITY;

@@ -13,14 +13,18 @@ Two independent restatements are kept side by side:
   ``linear + D0 (+ D1)`` (test_gemm_bias_broadcast.py:213-216,372-376),
   ``bmm(Q, K^T)`` (test_bmm.py:50-51),
   ``softmax(Q K^T * scale) V`` with the 0213 permute (test_bmm_softmax_bmm.py:90,111-114), and the
-  5-D output permutations of the permuting GEMMs (test_gemm_bias_permute.py:73-75,138-140).
+  5-D output permutations of the permuting GEMMs (test_gemm_bias_permute.py:73-75,138-140), and
+  attention on [batch, heads, seq, head_dim] operands with an optional key-padding mask from per-batch key
+  lengths (test_attention.py:504-523,593).
 * ``c_*`` — the plain-C triple loops of ``oracle/gemm_oracle.c`` (fp32 accumulate,
   optional reference rounding points), loaded through ctypes.
 
 Parity status: the reference ships no golden vectors for this path (its tests
 compare against PyTorch on a GPU), so every function here is pinned by closed
 forms, invariants and brute force in ``tests/test_oracle.py`` rather than by
-fixtures of the reference.
+fixtures of the reference.  One convention is pinned by nothing in the reference
+("parity unpinned"): ``torch_mem_eff_attention`` returns zeros for a batch entry
+whose key length is 0, where PyTorch's softmax gives NaN.
 """
 from __future__ import annotations
 
@@ -169,6 +173,30 @@ def torch_multihead_attention(x, qkv_w, qkv_b, proj_w, proj_b, residual, num_hea
     if residual is not None:
         y = y + _f(residual).reshape(B * S, D)
     return y.reshape(B, S, D)
+
+
+def torch_mem_eff_attention(q, k, v, causal: bool = False, lengths_kv=None) -> torch.Tensor:
+    """fp32 attention on [batch, heads, seq, head_dim] operands, result [batch, seq_q, heads, head_dim_v], scale
+    head_dim ** -0.5 (python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-263).  `lengths_kv` is the
+    key-padding mask of the reference's test (tests/unittest/ops/test_attention.py:504-523: key n of batch entry b
+    counts iff n < lengths_kv[b]).  A batch entry without keys is all zeros here, the kernel library's convention;
+    PyTorch's softmax gives NaN for it and the reference's test accepts either side's NaN only if both have it, so
+    that case is pinned by nothing in the reference."""
+    q, k, v = _f(q), _f(k), _f(v)
+    batch, heads, seq_q, d = q.shape
+    seq_kv = k.shape[2]
+    s = torch.matmul(q, k.transpose(-1, -2)) * (d ** -0.5)
+    dead = torch.zeros(batch, 1, seq_q, seq_kv, dtype=torch.bool)
+    if lengths_kv is not None:
+        lens = lengths_kv.detach().to("cpu").reshape(batch).long()
+        dead = dead | (torch.arange(seq_kv)[None, None, None, :] >= lens[:, None, None, None])
+    if causal:
+        dead = dead | torch.triu(torch.ones(seq_q, seq_kv, dtype=torch.bool), diagonal=1)[None, None]
+    s = s.masked_fill(dead, float("-inf"))
+    p = torch.softmax(s, dim=-1)
+    p = torch.where(torch.isnan(p), torch.zeros_like(p), p)  # rows with every key masked
+    v = torch.where(torch.isnan(v) | torch.isinf(v), torch.zeros_like(v), v)  # masked rows may hold anything
+    return torch.matmul(p, v).permute(0, 2, 1, 3).contiguous()
 
 
 def torch_cross_attention(q_in, k_in, v_in, wq, wk, wv, bq, bk, bv, proj_w, proj_b, residual, num_heads: int,

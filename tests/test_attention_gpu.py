@@ -123,6 +123,61 @@ def test_empty_keys_give_zero_and_empty_batch_is_noop():
         eager.bmm_softmax_bmm_permute(q, k, v, (3,))  # batch 2 is not a multiple of 3 heads
 
 
+def _check_mem_eff(batch, heads, S, Skv, d, dv, lens, causal=False, dtype=torch.float16, seed=0):
+    print(f"case mem_eff_attention batch={batch} heads={heads} S={S} Skv={Skv} d={d} dv={dv} lens={lens} "
+          f"causal={causal} {dtype}", flush=True)
+    q, k, v = (_rand(sh, dtype, seed + i)
+               for i, sh in enumerate(((batch, heads, S, d), (batch, heads, Skv, d), (batch, heads, Skv, dv))))
+    lengths = None if lens is None else torch.tensor(lens, dtype=torch.int32).reshape(batch, 1)
+    want = oracle.torch_mem_eff_attention(q, k, v, causal, lengths).to(dtype).float()
+    if lengths is not None:
+        # rows past a batch entry's length must not be read: poison them
+        for b in range(batch):
+            k[b, :, max(0, min(Skv, int(lens[b]))):] = float("nan")
+            v[b, :, max(0, min(Skv, int(lens[b]))):] = float("nan")
+    got = eager.mem_eff_attention(q.cuda(), k.cuda(), v.cuda(), causal=causal,
+                                  lengths_kv=None if lengths is None else lengths.cuda())
+    torch.cuda.synchronize()
+    assert got.shape == (batch, S, heads, dv)
+    torch.testing.assert_close(got.cpu().float(), want, atol=TOL, rtol=TOL)
+
+
+@pytest.mark.parametrize("mode", [None, 0, 1, 2, 3])
+@pytest.mark.parametrize("batch,heads,S,Skv,d,dv,lens,causal", [
+    (4, 2, 300, 1000, 40, 40, [1000, 517, 128, 1], False),   # whole tiles, a ragged last tile, one key
+    (4, 2, 300, 900, 40, 40, [900, 300, 77, 0], True),       # causal bound and key length, whichever is shorter
+    (3, 4, 70, 384, 32, 32, [384, 129, 0], False),           # a batch entry without keys is zeros
+    (2, 2, 40, 50, 40, 40, [50, 49], False),                 # single tile
+    (2, 3, 64, 200, 64, 128, [1200, -3], False),             # lengths are clamped to [0, Skv]
+])
+def test_mem_eff_attention_key_lengths(monkeypatch, mode, batch, heads, S, Skv, d, dv, lens, causal):
+    """Key lengths through the C ABI for every kernel variant (as in test_attention.py:504-523 of the reference)."""
+    if mode is not None:
+        monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+    _check_mem_eff(batch, heads, S, Skv, d, dv, lens, causal=causal, seed=Skv)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("batch,heads,S,Skv,d,dv,lens", [
+    (2, 8, 1024, 77, 40, 40, None),                          # fixed length: the cross-attention of a diffusion UNet
+    (2, 4, 197, 197, 64, 64, [197, 50]),
+    (3, 2, 50, 333, 20, 24, [333, 100, 7]),                  # head dims that are no multiple of 8: element-wise loads
+    (2, 2, 128, 256, 160, 160, [256, 65]),
+])
+def test_mem_eff_attention_shapes_and_dtypes(dtype, batch, heads, S, Skv, d, dv, lens):
+    _check_mem_eff(batch, heads, S, Skv, d, dv, lens, dtype=dtype, seed=d)
+
+
+def test_mem_eff_attention_argument_checks():
+    q = torch.randn(2, 2, 8, 16, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        eager.mem_eff_attention(q, q, q, lengths_kv=torch.zeros(2, dtype=torch.int64, device="cuda"))
+    with pytest.raises(ValueError):
+        eager.mem_eff_attention(q, q, q, lengths_kv=torch.zeros(3, dtype=torch.int32, device="cuda"))
+    with pytest.raises(ValueError):
+        eager.mem_eff_attention(q, q[:, :1], q)
+
+
 def test_config_c5_full_size():
     print("case config=c5 full size", flush=True)
     inp = oracle.config_inputs("c5")

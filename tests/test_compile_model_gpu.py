@@ -203,9 +203,38 @@ def test_mem_eff_attention_fixed_lengths(B, H, M, N, D, Dv, causal, copy_op):
     module.close()
 
 
-def test_mem_eff_attention_variable_lengths_are_refused():
-    with pytest.raises(NotImplementedError):
-        ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)
+@pytest.mark.parametrize("causal,var_q,copy_op", [(False, False, False), (True, False, True), (False, True, False)])
+def test_mem_eff_attention_variable_lengths(causal, var_q, copy_op):
+    """Key lengths (and, accepted but unspecified, query lengths) as the reference's test feeds them: [batch, 1] "int"
+    tensors; rows past a query length are blanked on both sides before comparing
+    (tests/unittest/ops/test_attention.py:504-523, 563-594, 661-664)."""
+    B, H, S, D = 4, 4, 300, 64
+    print(f"case compile_model mem_eff_attention lengths causal={causal} var_q={var_q}", flush=True)
+    Q = Tensor(shape=[B, H, S, D], dtype="float16", name="q", is_input=True)
+    K = Tensor(shape=[B, H, S, D], dtype="float16", name="k", is_input=True)
+    V = Tensor(shape=[B, H, S, D], dtype="float16", name="v", is_input=True)
+    L_kv = Tensor(shape=[B, 1], dtype="int", name="lengths_kv", is_input=True)
+    L_q = Tensor(shape=[B, 1], dtype="int", name="lengths_q", is_input=True) if var_q else None
+    OP = ops.mem_eff_attention(causal=causal, variable_seq_length_kv=True, variable_seq_length_q=var_q)
+    if copy_op:
+        OP = ops.mem_eff_attention(**OP._get_op_attributes())
+    Y = _mark_output(OP(Q, K, V, L_kv, L_q))
+    module = compile_model(Y, detect_target(), WORKDIR, f"mem_eff_attention_lengths_{next(_counter)}")
+    q, k, v = _rand((B, H, S, D), 1), _rand((B, H, S, D), 2), _rand((B, H, S, D), 3)
+    lengths_kv = torch.tensor([[300], [129], [1], [200]], dtype=torch.int32)
+    lengths_q = torch.tensor([[300], [10], [299], [0]], dtype=torch.int32)
+    feed = {"q": q.cuda(), "k": k.cuda(), "v": v.cuda(), "lengths_kv": lengths_kv.cuda()}
+    if var_q:
+        feed["lengths_q"] = lengths_q.cuda()
+    y = torch.empty(B, S, H, D, dtype=torch.float16, device="cuda")
+    module.run_with_tensors(feed, [y])
+    want = oracle.torch_mem_eff_attention(q, k, v, causal, lengths_kv).half().float()
+    got = y.cpu().float()
+    if var_q:
+        blank = (torch.arange(S)[None, :] >= lengths_q.long())[:, :, None, None]
+        got, want = got.masked_fill(blank, 0.0), want.masked_fill(blank, 0.0)
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+    module.close()
 
 
 @pytest.mark.parametrize("B,M,N,K,D,copy_op", [(24, 256, 256, 64, 64, False), (5, 100, 49, 40, 40, True)])

@@ -592,7 +592,8 @@ def test_mem_eff_attention_op_shapes_keys_and_hooks():
     op = ops.mem_eff_attention(causal=False)
     y = op(q, k, v)
     assert [d.value() for d in y.shape()] == [2, 64, 8, 48]
-    assert op._get_op_attributes() == {"causal": False}
+    assert op._get_op_attributes() == {"causal": False, "variable_seq_length_kv": False,
+                                       "variable_seq_length_q": False, "use_grouped_fmha": False}
     assert op._attrs["head_size"] == 48 and op._attrs["workspace"] == 0
     assert list(op._attrs["exec_path"]) == ["batch_size == 2 && num_heads == 8 && seq_len == 64 && head_sizes == 40"]
     op._attrs["name"] = "mem_eff_attention_0"
@@ -602,22 +603,38 @@ def test_mem_eff_attention_op_shapes_keys_and_hooks():
     y._attrs["name"] = "y"
     decl = registry.get("rocm.mem_eff_attention.func_decl")(op._attrs)
     assert decl.startswith("void mem_eff_attention_0(void* output, const void* q, const void* k, const void* v, "
-                           "int64_t* batch_size, int64_t* seq_len, int64_t* seq_len_kv, int num_heads, ")
+                           "const void* lengths_kv, int64_t* batch_size, int64_t* seq_len, int64_t* seq_len_kv, "
+                           "int num_heads, ")
     call = registry.get("rocm.mem_eff_attention.func_call")(op._attrs)
-    assert call == f"  mem_eff_attention_0(y, q, k, v, &q_dim_0, &q_dim_2, &k_dim_2, 8, 40, 48, {40 ** -0.5!r}f, stream);"
+    assert call == (f"  mem_eff_attention_0(y, q, k, v, nullptr, &q_dim_0, &q_dim_2, &k_dim_2, 8, 40, 48, "
+                    f"{40 ** -0.5!r}f, stream);")
     causal_op = ops.mem_eff_attention(causal=True)
     causal_op(q, k, v)
     causal_op._attrs["name"] = "mem_eff_attention_1"
     with detect_target():
         src = op.gen_function()
         causal_src = causal_op.gen_function()
-    assert "aitamd_bmm_softmax_bmm_permute(0, q, k, v, output, B, *seq_len, *seq_len_kv, head_dim, head_dim_v," in src
-    assert "num_heads, softmax_scale, 0, stream)" in src
-    assert "num_heads, softmax_scale, 1, stream)" in causal_src
-    with pytest.raises(NotImplementedError):
-        ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)
-    with pytest.raises(NotImplementedError):
-        ops.mem_eff_attention(causal=False)(q, k, v, lengths_kv=Tensor([2], name="len", dtype="int32", is_input=True))
+    assert ("aitamd_mem_eff_attention(0, q, k, v, output, *batch_size, num_heads, *seq_len, *seq_len_kv, head_dim,"
+            in src)
+    assert "head_dim_v, softmax_scale, 0," in src and "head_dim_v, softmax_scale, 1," in causal_src
+    # key lengths: a fourth (and, for query lengths, fifth) input of dtype "int"; only the key lengths reach the kernel
+    var = ops.mem_eff_attention(causal=False, variable_seq_length_kv=True, variable_seq_length_q=True)
+    lens_kv = Tensor([2, 1], name="lens_kv", dtype="int", is_input=True)
+    lens_q = Tensor([2, 1], name="lens_q", dtype="int", is_input=True)
+    y2 = var(q, k, v, lens_kv, lens_q)
+    assert [t._attrs["name"] for t in var._attrs["inputs"]] == ["q", "k", "v", "lens_kv", "lens_q"]
+    assert lens_kv._attrs["dtype"] == "int32"
+    var._attrs["name"] = "mem_eff_attention_2"
+    y2._attrs["name"] = "y2"
+    assert registry.get("rocm.mem_eff_attention.func_call")(var._attrs).startswith(
+        "  mem_eff_attention_2(y2, q, k, v, lens_kv, &q_dim_0,")
+    copy = ops.mem_eff_attention(**var._get_op_attributes())
+    assert copy._attrs["variable_seq_length_kv"] and copy._attrs["variable_seq_length_q"]
+    with pytest.raises(AssertionError):
+        ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)(q, k, v)
+    with pytest.raises(RuntimeError, match="int32"):
+        ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)(
+            q, k, v, Tensor([2, 1], name="bad", dtype="float16", is_input=True))
     with pytest.raises(RuntimeError, match="head dims"):
         ops.mem_eff_attention(causal=False)(q, Tensor([2, 8, 77, 32], name="k2", is_input=True), v)
 

@@ -278,6 +278,55 @@ def test_attention_block_matches_torch_nn_multiheadattention(causal):
     assert torch.allclose(got, want + res.reshape(B, S, D), atol=1e-5)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_cross_attention_block_matches_torch_nn_multiheadattention(causal):
+    """Separate q / k / v projections are the three row blocks of the library module's packed in_proj."""
+    B, S, Skv, D, H = 2, 7, 7 if causal else 5, 16, 4
+    mha = torch.nn.MultiheadAttention(D, H, bias=True, batch_first=True).eval()
+    q, k, v = (_rand((B, n, D), torch.float32, seed=6 + i) for i, n in enumerate((S, Skv, Skv)))
+    res = _rand((B * S, D), torch.float32, seed=9)
+    wq, wk, wv = mha.in_proj_weight.chunk(3)
+    bq, bk, bv = mha.in_proj_bias.chunk(3)
+    mask = torch.triu(torch.ones(S, Skv, dtype=torch.bool), diagonal=1) if causal else None
+    with torch.no_grad():
+        want, _ = mha(q, k, v, attn_mask=mask, need_weights=False)
+        got = oracle.torch_cross_attention(q, k, v, wq, wk, wv, bq, bk, bv, mha.out_proj.weight, mha.out_proj.bias,
+                                           res, H, causal)
+    assert torch.allclose(got, want + res.reshape(B, S, D), atol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_mem_eff_attention_key_lengths(causal):
+    """Three pins: without lengths it is the pinned bmm_softmax_bmm_permute on [batch * heads] operands; with
+    lengths every batch entry equals the fixed-length result on its truncated keys (rows past the length may hold
+    anything, NaN included); and it agrees with the library's scaled_dot_product_attention under a padding mask."""
+    batch, heads, S, Skv, d, dv = 3, 2, 9, 11, 8, 6
+    q, k, v = (_rand(sh, torch.float32, seed=20 + i)
+               for i, sh in enumerate(((batch, heads, S, d), (batch, heads, Skv, d), (batch, heads, Skv, dv))))
+    flat = oracle.torch_bmm_softmax_bmm_permute(q.reshape(-1, S, d), k.reshape(-1, Skv, d), v.reshape(-1, Skv, dv),
+                                                d ** -0.5, heads, causal)
+    assert torch.allclose(oracle.torch_mem_eff_attention(q, k, v, causal), flat, atol=1e-6)
+    lens = torch.tensor([[11], [4], [1]], dtype=torch.int32)
+    k2, v2 = k.clone(), v.clone()
+    for b in range(batch):
+        k2[b, :, int(lens[b]):] = float("nan")
+        v2[b, :, int(lens[b]):] = float("nan")
+    got = oracle.torch_mem_eff_attention(q, torch.nan_to_num(k2, nan=7.0), v2, causal, lens)
+    for b in range(batch):
+        n = int(lens[b])
+        want = oracle.torch_mem_eff_attention(q[b:b + 1], k[b:b + 1, :, :n], v[b:b + 1, :, :n], causal)
+        assert torch.allclose(got[b:b + 1], want, atol=1e-6)
+    keep = torch.arange(Skv)[None, :] < lens.long()                       # [batch, Skv]
+    mask = keep[:, None, None, :].expand(batch, 1, S, Skv)
+    if causal:
+        mask = mask & torch.tril(torch.ones(S, Skv, dtype=torch.bool))
+    sdpa = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask).permute(0, 2, 1, 3)
+    assert torch.allclose(oracle.torch_mem_eff_attention(q, k, v, causal, lens), sdpa, atol=1e-5)
+    # no keys at all: zeros by this library's convention
+    zero = oracle.torch_mem_eff_attention(q, k, v, causal, torch.zeros(batch, 1, dtype=torch.int32))
+    assert torch.count_nonzero(zero) == 0
+
+
 def test_bmm_rcr_permute_places_each_batch_as_a_head():
     """out[g, m, h, n] must be (Q[g*d1 + h] @ K[g*d1 + h]^T)[m, n]: brute force over the batch index."""
     B, M, N, K, d1 = 6, 5, 7, 4, 3

@@ -103,3 +103,41 @@ def test_attention_random_shapes(monkeypatch):
         torch.cuda.synchronize()
         ok, err = _close(got, want, 2e-2 if dtype == torch.float16 else 4e-2)
         assert ok, f"case {i}: max error {err}"
+
+
+def test_mem_eff_attention_random_shapes_and_key_lengths(monkeypatch):
+    rng = random.Random(4321)
+    for i in range(100):
+        heads = rng.choice([1, 2, 4, 8])
+        batch = rng.choice([1, 2, 3, 5])
+        S = rng.choice([1, 31, 33, 100, 128, 129, 256, 300, 511])
+        Skv = rng.choice([1, 5, 33, 64, 77, 127, 128, 129, 200, 256, 300, 383, 500, 777, 1024])
+        d = rng.choice([8, 16, 20, 32, 40, 64, 96, 128, 160])
+        dv = rng.choice([8, 16, 24, 40, 64, 128, 160])
+        causal = rng.random() < 0.3
+        dtype = torch.float16 if rng.random() < 0.7 else torch.bfloat16
+        mode = rng.choice([None, 0, 1, 2, 3])
+        if mode is None:
+            monkeypatch.delenv("AITAMD_ATTN_MODE", raising=False)
+        else:
+            monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+        lens = None
+        if rng.random() < 0.8:
+            lens = torch.tensor([rng.choice([0, 1, Skv, Skv // 2, rng.randint(0, Skv)]) for _ in range(batch)],
+                                dtype=torch.int32)
+        g = torch.Generator().manual_seed(1000 + i)
+        q = torch.randn(batch, heads, S, d, generator=g).to(dtype)
+        k = torch.randn(batch, heads, Skv, d, generator=g).to(dtype)
+        v = torch.randn(batch, heads, Skv, dv, generator=g).to(dtype)
+        print(f"case {i} mem_eff_attention batch={batch} heads={heads} S={S} Skv={Skv} d={d} dv={dv} causal={causal} "
+              f"{dtype} mode={mode} lens={None if lens is None else lens.tolist()}", flush=True)
+        want = oracle.torch_mem_eff_attention(q, k, v, causal, lens).to(dtype).float()
+        if lens is not None:
+            for b in range(batch):  # rows past the length must not be read
+                k[b, :, int(lens[b]):] = float("nan")
+                v[b, :, int(lens[b]):] = float("nan")
+        got = eager.mem_eff_attention(q.cuda(), k.cuda(), v.cuda(), causal=causal,
+                                      lengths_kv=None if lens is None else lens.cuda())
+        torch.cuda.synchronize()
+        ok, err = _close(got, want, 2e-2 if dtype == torch.float16 else 4e-2)
+        assert ok, f"case {i}: max error {err}"
