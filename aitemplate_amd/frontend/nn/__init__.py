@@ -1,4 +1,4 @@
-from .attention import CrossAttention, MultiheadAttention  # noqa: F401
+from .attention import CrossAttention, ScaledDotProductAttention, MultiheadAttention  # noqa: F401
 from .dropout import Dropout, DropPath  # noqa: F401
 from .linear import Linear  # noqa: F401
 from .module import Module  # noqa: F401

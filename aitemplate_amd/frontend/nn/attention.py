@@ -131,3 +131,14 @@ class CrossAttention(Module):
             x = self.proj(attn_output)
         x = self.proj_drop(x)
         return ops.reshape()(x, [batch, seq, self.dim])
+
+
+class ScaledDotProductAttention(Module):
+    """softmax(q k^T / sqrt(head_dim)) v on [batch, heads, seq, head_dim] operands, result [batch, seq, heads, head_dim]
+    (python/aitemplate/frontend/nn/attention.py:403-410)."""
+
+    def __init__(self) -> None:
+        super().__init__()
+
+    def forward(self, q, k, v):
+        return ops.mem_eff_attention(causal=False)(q, k, v)

@@ -189,6 +189,10 @@ def test_mem_eff_attention_fixed_lengths(B, H, M, N, D, Dv, causal, copy_op):
     OP = ops.mem_eff_attention(causal=causal)
     if copy_op:
         OP = ops.mem_eff_attention(**OP._get_op_attributes())
+    if not causal and not copy_op:
+        from aitemplate_amd.frontend import nn
+
+        OP = nn.ScaledDotProductAttention()   # the module form of the same op (frontend/nn/attention.py:403-410)
     Y = _mark_output(OP(Q, K, V))
     module = compile_model(Y, detect_target(), WORKDIR, f"mem_eff_attention_{next(_counter)}")
     q, k, v = _rand((B, H, M, D), 1), _rand((B, H, N, D), 2), _rand((B, H, N, Dv), 3)
