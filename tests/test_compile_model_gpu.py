@@ -241,6 +241,28 @@ def test_mem_eff_attention_variable_lengths(causal, var_q, copy_op):
     module.close()
 
 
+def test_mem_eff_attention_dynamic_batch_and_sequence_bf16():
+    """One library for batch in [1, 4] and query / key sequences in [64, 256], bf16, with key lengths."""
+    H, D = 4, 64
+    batch = shape_utils.gen_int_var_min_max([1, 4], name="batch_size")
+    seq = shape_utils.gen_int_var_min_max([64, 256], name="seq")
+    Q = Tensor(shape=[batch, H, seq, D], dtype="bfloat16", name="q", is_input=True)
+    K = Tensor(shape=[batch, H, seq, D], dtype="bfloat16", name="k", is_input=True)
+    V = Tensor(shape=[batch, H, seq, D], dtype="bfloat16", name="v", is_input=True)
+    L = Tensor(shape=[batch, 1], dtype="int", name="lengths_kv", is_input=True)
+    Y = _mark_output(ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)(Q, K, V, L))
+    module = compile_model(Y, detect_target(), WORKDIR, f"mem_eff_attention_dynamic_{next(_counter)}")
+    for b, s_len in ((1, 64), (4, 256), (3, 100)):
+        print(f"case compile_model mem_eff_attention dynamic batch={b} seq={s_len}", flush=True)
+        q, k, v = (_rand((b, H, s_len, D), i, dtype=torch.bfloat16) for i in (1, 2, 3))
+        lens = torch.tensor([[s_len], [s_len // 3], [1], [s_len - 1]][:b], dtype=torch.int32)
+        y = torch.empty(b, s_len, H, D, dtype=torch.bfloat16, device="cuda")
+        module.run_with_tensors({"q": q.cuda(), "k": k.cuda(), "v": v.cuda(), "lengths_kv": lens.cuda()}, [y])
+        want = oracle.torch_mem_eff_attention(q, k, v, False, lens).bfloat16().float()
+        torch.testing.assert_close(y.cpu().float(), want, atol=4e-2, rtol=4e-2)
+    module.close()
+
+
 @pytest.mark.parametrize("B,M,N,K,D,copy_op", [(24, 256, 256, 64, 64, False), (5, 100, 49, 40, 40, True)])
 def test_bmm_softmax_bmm(B, M, N, K, D, copy_op):   # the non-permuted op (reference: test_bmm_softmax_bmm.py:59-118)
     X = Tensor(shape=[B, M, K], name="input_0", is_input=True)
