@@ -48,6 +48,9 @@ class mem_eff_attention(Operator):
                 raise RuntimeError("mem_eff_attention: the number of heads and the head dim must be static")
         if q._attrs["shape"][3] != k._attrs["shape"][3] or k._attrs["shape"][2] != v._attrs["shape"][2]:
             raise RuntimeError("mem_eff_attention: q / k head dims and k / v sequence lengths must agree")
+        for t, name in ((k, "k"), (v, "v")):
+            if t._attrs["shape"][0] != q._attrs["shape"][0] or t._attrs["shape"][1] != q._attrs["shape"][1]:
+                raise RuntimeError(f"mem_eff_attention: batch and heads of {name} differ from q's")
         self._attrs["head_size"] = v._attrs["shape"][3]._attrs["values"][0]
         self._attrs["inputs"] = [q, k, v]
         for flag, lengths, name in ((self._attrs["variable_seq_length_kv"], lengths_kv, "lengths_kv"),
@@ -56,6 +59,9 @@ class mem_eff_attention(Operator):
                 assert lengths is not None, f"mem_eff_attention: {name} is required"
                 if lengths._attrs["dtype"] != "int32":
                     raise RuntimeError(f"mem_eff_attention: {name} must be int32, got {lengths._attrs['dtype']}")
+                lshape = lengths._attrs["shape"]
+                if lshape[0] != q._attrs["shape"][0] or any(d._attrs["values"] != [1] for d in lshape[1:]):
+                    raise RuntimeError(f"mem_eff_attention: {name} must hold one entry per batch ([batch] or [batch, 1])")
                 self._attrs["inputs"].append(lengths)
         self._set_depth()
         self._extract_exec_path(q)

@@ -632,6 +632,11 @@ def test_mem_eff_attention_op_shapes_keys_and_hooks():
     assert copy._attrs["variable_seq_length_kv"] and copy._attrs["variable_seq_length_q"]
     with pytest.raises(AssertionError):
         ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)(q, k, v)
+    with pytest.raises(RuntimeError, match="one entry per batch"):
+        ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)(
+            q, k, v, Tensor([3, 1], name="bad_len", dtype="int", is_input=True))
+    with pytest.raises(RuntimeError, match="batch and heads"):
+        ops.mem_eff_attention(causal=False)(q, Tensor([2, 4, 77, 40], name="k4", is_input=True), v)
     with pytest.raises(RuntimeError, match="int32"):
         ops.mem_eff_attention(causal=False, variable_seq_length_kv=True)(
             q, k, v, Tensor([2, 1], name="bad", dtype="float16", is_input=True))
