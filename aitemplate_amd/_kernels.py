@@ -144,7 +144,7 @@ def load() -> ctypes.CDLL:
                                                        ctypes.c_float, i32, vp]
         lib.aitamd_mem_eff_attention.restype = i32
         lib.aitamd_mem_eff_attention.argtypes = [i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, i32,
-                                                 vp, vp]
+                                                 vp, vp, vp]
         _lib = lib
         return lib
 

@@ -4,8 +4,8 @@ Takes the place of python/aitemplate/backend/rocm/attention/mem_eff_attention.py
 `func_decl`, `func_call` under the same registry keys).  [batch, heads, seq, head_dim] operands are the
 [batch * heads, seq, head_dim] operands of the fused attention kernel, and the op's [batch, seq, heads, head_dim_v]
 result is that kernel's permuted store with heads as the group size, so the launcher is one call; the scale is
-head_dim ** -0.5 as the reference passes it (mem_eff_attention.py:343).  Key lengths stay on the device: the kernel
-reads its batch entry's length itself (the reference's hook copies nothing either but dereferences the device pointer
+head_dim ** -0.5 as the reference passes it (mem_eff_attention.py:343).  Key and query lengths stay on the device: the kernel
+reads its batch entry's lengths itself (the reference's hook copies nothing either but dereferences the device pointer
 on the host, mem_eff_attention.py:181-182)."""
 from typing import Any, Dict
 
@@ -15,7 +15,7 @@ from ..gemm import common
 
 def _signature(func_name: str) -> str:
     return (f"void {func_name}(void* output, const void* q, const void* k, const void* v, const void* lengths_kv, "
-            "int64_t* batch_size, int64_t* seq_len, int64_t* seq_len_kv, int num_heads, int head_dim, "
+            "const void* lengths_q, int64_t* batch_size, int64_t* seq_len, int64_t* seq_len_kv, int num_heads, int head_dim, "
             "int head_dim_v, float softmax_scale, hipStream_t stream)")
 
 
@@ -27,7 +27,8 @@ def gen_function(func_attrs: Dict[str, Any]) -> str:
 {_signature(func_name)} {{
   check_rc(aitamd_mem_eff_attention({dtype}, q, k, v, output, *batch_size, num_heads, *seq_len, *seq_len_kv, head_dim,
                                     head_dim_v, softmax_scale, {causal},
-                                    static_cast<const int32_t*>(lengths_kv), stream), "{func_name}");
+                                    static_cast<const int32_t*>(lengths_kv), static_cast<const int32_t*>(lengths_q),
+                                    stream), "{func_name}");
 }}
 {common.FOOTER}"""
 
@@ -38,14 +39,16 @@ def func_decl(func_attrs: Dict[str, Any]) -> str:
 
 def func_call(func_attrs: Dict[str, Any], indent: str = "  ") -> str:
     q, k, v = func_attrs["inputs"][:3]
-    lengths_kv = func_attrs["inputs"][3]._attrs["name"] if func_attrs["variable_seq_length_kv"] else "nullptr"
+    extra = [t._attrs["name"] for t in func_attrs["inputs"][3:]]  # lengths_kv, then lengths_q, each if its flag is set
+    lengths_kv = extra.pop(0) if func_attrs["variable_seq_length_kv"] else "nullptr"
+    lengths_q = extra.pop(0) if func_attrs["variable_seq_length_q"] else "nullptr"
     out = func_attrs["outputs"][0]
     qs, ks, vs = q._attrs["shape"], k._attrs["shape"], v._attrs["shape"]
     heads = qs[1]._attrs["values"][0]
     head_dim = qs[3]._attrs["values"][0]
     head_dim_v = vs[3]._attrs["values"][0]
     scale = head_dim ** (-0.5)
-    args = [out._attrs["name"], q._attrs["name"], k._attrs["name"], v._attrs["name"], lengths_kv, "&" + qs[0]._attrs["name"],
+    args = [out._attrs["name"], q._attrs["name"], k._attrs["name"], v._attrs["name"], lengths_kv, lengths_q, "&" + qs[0]._attrs["name"],
             "&" + qs[2]._attrs["name"], "&" + ks[2]._attrs["name"], str(heads), str(head_dim), str(head_dim_v),
             f"{scale!r}f", "stream"]
     return f"{indent}{func_attrs['name']}({', '.join(args)});"

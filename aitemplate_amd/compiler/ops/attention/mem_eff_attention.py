@@ -6,8 +6,8 @@ Counterpart of python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-
 reference's ROCm hook (backend/rocm/attention/mem_eff_attention.py) reads the device-side lengths on the host and is
 skipped by its own test on ROCm (tests/unittest/ops/test_attention.py:705); the meaning built here is the one that
 test states for every backend (test_attention.py:504-523, 593, 661-664): `lengths_kv` [batch, 1] int32 is a key-padding
-mask (batch entry b attends to its first lengths_kv[b] keys), rows past `lengths_q` are unspecified, so `lengths_q` is
-accepted and not read.  `nn.CrossAttention` uses the fixed-length form (frontend/nn/attention.py:338).
+mask (batch entry b attends to its first lengths_kv[b] keys); rows past `lengths_q` are unspecified there and are
+written as zeros here (blocks of query rows that are all padding do no work).  `nn.CrossAttention` uses the fixed-length form (frontend/nn/attention.py:338).
 `use_grouped_fmha` selects between two CUDA kernels in the reference and changes nothing here."""
 import itertools
 from collections import OrderedDict

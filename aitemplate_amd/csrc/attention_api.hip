@@ -103,7 +103,7 @@ namespace {
 
 int attention_entry(const char* who, int dtype, const void* q, const void* k, const void* v, void* out, int64_t B,
                     int64_t M, int64_t N, int64_t K, int64_t O, int64_t G, float scale, int causal,
-                    const int32_t* kv_len, void* stream) {
+                    const int32_t* kv_len, const int32_t* q_len, void* stream) {
   if (dtype != 0 && dtype != 1) return fail("%s: bad dtype %d", who, dtype);
   if (B < 0 || M < 0 || N < 0 || K < 0 || O < 0) return fail("%s: negative dimension", who);
   if (G <= 0 || (B % G) != 0) return fail("%s: batch %lld is not a multiple of heads %lld", who,
@@ -129,6 +129,7 @@ int attention_entry(const char* who, int dtype, const void* q, const void* k, co
   p.scale_log2e = round_to_elem(scale, dtype) * 1.4426950408889634f;
   p.causal = causal ? 1 : 0;
   p.kv_len = kv_len;
+  p.q_len = q_len;
   const int ks = (int)((K + 15) / 16) > 0 ? (int)((K + 15) / 16) : 1;
   const int ot = (int)((O + 31) / 32);
   const bool vec = (K % 8 == 0) && (O % 8 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15) == 0) &&
@@ -181,16 +182,16 @@ extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const vo
                                               int64_t B, int64_t M, int64_t N, int64_t K, int64_t O, int64_t G,
                                               float scale, int causal, void* stream) {
   return attention_entry("aitamd_bmm_softmax_bmm_permute", dtype, q, k, v, out, B, M, N, K, O, G, scale, causal, nullptr,
-                         stream);
+                         nullptr, stream);
 }
 
 extern "C" int aitamd_mem_eff_attention(int dtype, const void* q, const void* k, const void* v, void* out,
                                         int64_t batch, int64_t heads, int64_t seq_q, int64_t seq_kv, int64_t head_dim,
                                         int64_t head_dim_v, float scale, int causal, const int32_t* lengths_kv,
-                                        void* stream) {
+                                        const int32_t* lengths_q, void* stream) {
   if (batch < 0 || heads <= 0) return fail("aitamd_mem_eff_attention: bad batch %lld or heads %lld", (long long)batch,
                                            (long long)heads);
   if (batch > 0x7fffffffll / heads) return fail("aitamd_mem_eff_attention: dimension too large");
   return attention_entry("aitamd_mem_eff_attention", dtype, q, k, v, out, batch * heads, seq_q, seq_kv, head_dim,
-                         head_dim_v, heads, scale, causal, lengths_kv, stream);
+                         head_dim_v, heads, scale, causal, lengths_kv, lengths_q, stream);
 }

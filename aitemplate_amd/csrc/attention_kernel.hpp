@@ -45,6 +45,9 @@ struct AttnParams {
   // Optional, device memory, B / G entries: batch entry b only attends to its first kv_len[b / G] keys (clamped to
   // [0, N]); the later rows of K and V are never read.  Null: all N keys.
   const int32_t* kv_len;
+  // Optional, same form: rows m >= q_len[b / G] of batch entry b are written as zeros, and a workgroup whose rows
+  // all lie past that length visits no keys.
+  const int32_t* q_len;
 };
 
 // NW_ waves (32 query rows each) share the K / V tiles; NS_ LDS stages.  The register-staged
@@ -200,6 +203,12 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     if (p.kv_len != nullptr) {
       const int len = __builtin_amdgcn_readfirstlane(p.kv_len[b / p.G]);
       N = len < 0 ? 0 : (len < N ? len : N);
+    }
+    int m_rows = p.M;
+    if (p.q_len != nullptr) {
+      const int len = __builtin_amdgcn_readfirstlane(p.q_len[b / p.G]);
+      m_rows = len < 0 ? 0 : (len < m_rows ? len : m_rows);
+      if (m0 >= m_rows) N = 0;  // nothing but padding rows here: no keys, zeros out
     }
 
     // ---- Q fragments (B operand of S^T = K Q^T): lane (q = r32, k = 16 ks + 8 h + j)
@@ -540,7 +549,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
 
     // ---- normalise and store permuted: out[b / G][m][b % G][o]
     const float l_tot = sum_across_halves(l_run);
-    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    const float inv = (l_tot > 0.0f && q_row < m_rows) ? 1.0f / l_tot : 0.0f;
     if (q_row < p.M && grp == 0) {
       T* orow = reinterpret_cast<T*>(p.out) + (((int64_t)(b / p.G) * p.M + q_row) * p.G + (b % p.G)) * p.O;
       const bool vec_ok = ((p.O & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 7) == 0);

@@ -282,10 +282,12 @@ def bmm_softmax_bmm_permute(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, s
 
 
 def mem_eff_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool = False,
-                      lengths_kv: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      lengths_kv: Optional[torch.Tensor] = None, lengths_q: Optional[torch.Tensor] = None,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """softmax(q k^T / sqrt(head_dim)) v on [batch, heads, seq, head_dim] operands, written as
     [batch, seq_q, heads, head_dim_v]; `lengths_kv` ([batch] or [batch, 1], int32, on the device) limits batch entry b
-    to its first lengths_kv[b] keys (python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-263)."""
+    to its first lengths_kv[b] keys; `lengths_q`, same form, zeroes the query rows past lengths_q[b]
+    (python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-263)."""
     lib = _kernels.load()
     dtype = q.dtype
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
@@ -298,14 +300,14 @@ def mem_eff_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal:
     seq_kv, head_dim_v = v.shape[2], v.shape[3]
     if k.shape != (batch, heads, seq_kv, head_dim) or v.shape[:2] != (batch, heads):
         raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
-    if lengths_kv is not None:
-        if lengths_kv.dtype != torch.int32 or lengths_kv.numel() != batch or not lengths_kv.is_contiguous() \
-                or lengths_kv.device != q.device:
-            raise ValueError("lengths_kv must be a contiguous int32 tensor with one entry per batch on the operands' device")
+    for lengths, name in ((lengths_kv, "lengths_kv"), (lengths_q, "lengths_q")):
+        if lengths is not None and (lengths.dtype != torch.int32 or lengths.numel() != batch
+                                    or not lengths.is_contiguous() or lengths.device != q.device):
+            raise ValueError(f"{name} must be a contiguous int32 tensor with one entry per batch on the operands' device")
     if out is None:
         out = torch.empty(batch, seq_q, heads, head_dim_v, dtype=dtype, device=q.device)
     rc = lib.aitamd_mem_eff_attention(_TORCH_DTYPE_ID[dtype], _p(q), _p(k), _p(v), _p(out), batch, heads, seq_q, seq_kv,
                                       head_dim, head_dim_v, float(head_dim) ** -0.5, int(bool(causal)),
-                                      _p(lengths_kv) if lengths_kv is not None else None, _stream_ptr())
+                                      _p(lengths_kv), _p(lengths_q), _stream_ptr())
     _kernels.check(rc, "mem_eff_attention")
     return out

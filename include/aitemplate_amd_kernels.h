@@ -206,15 +206,16 @@ AITAMD_API int aitamd_bmm_softmax_bmm_permute(int dtype,
  * B = batch * heads and G = heads.  lengths_kv: null, or device memory with `batch` int32 entries: batch entry b
  * attends to its first lengths_kv[b] keys only (clamped to [0, seq_kv]; later rows of k and v are not read), the
  * key-padding mask of the reference's own test (tests/unittest/ops/test_attention.py:504-523, 593).  A batch entry
- * with no keys is written as zeros.  Query lengths need no argument: rows past a query length are unspecified in the
- * reference (its test blanks them on both sides, test_attention.py:661-664) and are computed like any other row.
+ * with no keys is written as zeros.  lengths_q: null, or the same form for query rows: rows m >= lengths_q[b] are
+ * written as zeros and blocks of query rows that are all padding visit no keys (the reference leaves such rows
+ * unspecified; its test blanks them on both sides, test_attention.py:661-664).
  * Replaces the op function that python/aitemplate/backend/rocm/attention/mem_eff_attention.py:305-365 renders
  * (frontend python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-263). */
 AITAMD_API int aitamd_mem_eff_attention(int dtype,
                                         const void* q, const void* k, const void* v, void* out,
                                         int64_t batch, int64_t heads, int64_t seq_q, int64_t seq_kv,
                                         int64_t head_dim, int64_t head_dim_v, float scale, int causal,
-                                        const int32_t* lengths_kv, void* stream);
+                                        const int32_t* lengths_kv, const int32_t* lengths_q, void* stream);
 
 #ifdef __cplusplus
 } /* extern "C" */

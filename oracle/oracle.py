@@ -24,7 +24,8 @@ compare against PyTorch on a GPU), so every function here is pinned by closed
 forms, invariants and brute force in ``tests/test_oracle.py`` rather than by
 fixtures of the reference.  One convention is pinned by nothing in the reference
 ("parity unpinned"): ``torch_mem_eff_attention`` returns zeros for a batch entry
-whose key length is 0, where PyTorch's softmax gives NaN.
+whose key length is 0, where PyTorch's softmax gives NaN, and zeros for query
+rows past a query length, which the reference leaves unspecified.
 """
 from __future__ import annotations
 
@@ -175,13 +176,14 @@ def torch_multihead_attention(x, qkv_w, qkv_b, proj_w, proj_b, residual, num_hea
     return y.reshape(B, S, D)
 
 
-def torch_mem_eff_attention(q, k, v, causal: bool = False, lengths_kv=None) -> torch.Tensor:
+def torch_mem_eff_attention(q, k, v, causal: bool = False, lengths_kv=None, lengths_q=None) -> torch.Tensor:
     """fp32 attention on [batch, heads, seq, head_dim] operands, result [batch, seq_q, heads, head_dim_v], scale
     head_dim ** -0.5 (python/aitemplate/compiler/ops/attention/mem_eff_attention.py:49-263).  `lengths_kv` is the
     key-padding mask of the reference's test (tests/unittest/ops/test_attention.py:504-523: key n of batch entry b
     counts iff n < lengths_kv[b]).  A batch entry without keys is all zeros here, the kernel library's convention;
     PyTorch's softmax gives NaN for it and the reference's test accepts either side's NaN only if both have it, so
-    that case is pinned by nothing in the reference."""
+    that case is pinned by nothing in the reference.  `lengths_q`: query rows m >= lengths_q[b] are zeros, again the
+    library's convention for rows the reference leaves unspecified (its test blanks them, test_attention.py:661-664)."""
     q, k, v = _f(q), _f(k), _f(v)
     batch, heads, seq_q, d = q.shape
     seq_kv = k.shape[2]
@@ -196,7 +198,11 @@ def torch_mem_eff_attention(q, k, v, causal: bool = False, lengths_kv=None) -> t
     p = torch.softmax(s, dim=-1)
     p = torch.where(torch.isnan(p), torch.zeros_like(p), p)  # rows with every key masked
     v = torch.where(torch.isnan(v) | torch.isinf(v), torch.zeros_like(v), v)  # masked rows may hold anything
-    return torch.matmul(p, v).permute(0, 2, 1, 3).contiguous()
+    out = torch.matmul(p, v).permute(0, 2, 1, 3).contiguous()  # [batch, seq_q, heads, head_dim_v]
+    if lengths_q is not None:
+        lq = lengths_q.detach().to("cpu").reshape(batch).long()
+        out = out.masked_fill((torch.arange(seq_q)[None, :] >= lq[:, None])[:, :, None, None], 0.0)
+    return out
 
 
 def torch_cross_attention(q_in, k_in, v_in, wq, wk, wv, bq, bk, bv, proj_w, proj_b, residual, num_heads: int,

@@ -123,20 +123,23 @@ def test_empty_keys_give_zero_and_empty_batch_is_noop():
         eager.bmm_softmax_bmm_permute(q, k, v, (3,))  # batch 2 is not a multiple of 3 heads
 
 
-def _check_mem_eff(batch, heads, S, Skv, d, dv, lens, causal=False, dtype=torch.float16, seed=0):
+def _check_mem_eff(batch, heads, S, Skv, d, dv, lens, causal=False, dtype=torch.float16, seed=0, lens_q=None):
     print(f"case mem_eff_attention batch={batch} heads={heads} S={S} Skv={Skv} d={d} dv={dv} lens={lens} "
           f"causal={causal} {dtype}", flush=True)
     q, k, v = (_rand(sh, dtype, seed + i)
                for i, sh in enumerate(((batch, heads, S, d), (batch, heads, Skv, d), (batch, heads, Skv, dv))))
     lengths = None if lens is None else torch.tensor(lens, dtype=torch.int32).reshape(batch, 1)
-    want = oracle.torch_mem_eff_attention(q, k, v, causal, lengths).to(dtype).float()
+    lengths_q = None if lens_q is None else torch.tensor(lens_q, dtype=torch.int32)
+    want = oracle.torch_mem_eff_attention(q, k, v, causal, lengths, lengths_q).to(dtype).float()
     if lengths is not None:
         # rows past a batch entry's length must not be read: poison them
         for b in range(batch):
             k[b, :, max(0, min(Skv, int(lens[b]))):] = float("nan")
             v[b, :, max(0, min(Skv, int(lens[b]))):] = float("nan")
     got = eager.mem_eff_attention(q.cuda(), k.cuda(), v.cuda(), causal=causal,
-                                  lengths_kv=None if lengths is None else lengths.cuda())
+                                  lengths_kv=None if lengths is None else lengths.cuda(),
+                                  lengths_q=None if lengths_q is None else lengths_q.cuda(),
+                                  out=torch.full((batch, S, heads, dv), 3.0, dtype=dtype, device="cuda"))
     torch.cuda.synchronize()
     assert got.shape == (batch, S, heads, dv)
     torch.testing.assert_close(got.cpu().float(), want, atol=TOL, rtol=TOL)
@@ -166,6 +169,16 @@ def test_mem_eff_attention_key_lengths(monkeypatch, mode, batch, heads, S, Skv, 
 ])
 def test_mem_eff_attention_shapes_and_dtypes(dtype, batch, heads, S, Skv, d, dv, lens):
     _check_mem_eff(batch, heads, S, Skv, d, dv, lens, dtype=dtype, seed=d)
+
+
+@pytest.mark.parametrize("mode", [None, 0, 1, 2, 3])
+@pytest.mark.parametrize("causal", [False, True])
+def test_mem_eff_attention_query_lengths(monkeypatch, mode, causal):
+    """Rows past a query length are zeros (whole blocks of them visit no keys), the rows before are unchanged."""
+    if mode is not None:
+        monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+    _check_mem_eff(5, 2, 700, 640, 40, 40, [640, 300, 640, 1, 640], causal=causal, seed=mode or 9,
+                   lens_q=[700, 130, 0, 257, 9000])
 
 
 def test_mem_eff_attention_argument_checks():

@@ -209,8 +209,8 @@ def test_mem_eff_attention_fixed_lengths(B, H, M, N, D, Dv, causal, copy_op):
 
 @pytest.mark.parametrize("causal,var_q,copy_op", [(False, False, False), (True, False, True), (False, True, False)])
 def test_mem_eff_attention_variable_lengths(causal, var_q, copy_op):
-    """Key lengths (and, accepted but unspecified, query lengths) as the reference's test feeds them: [batch, 1] "int"
-    tensors; rows past a query length are blanked on both sides before comparing
+    """Key and query lengths as the reference's test feeds them: [batch, 1] "int" tensors; the reference's test blanks
+    rows past a query length on both sides before comparing, here they are zeros
     (tests/unittest/ops/test_attention.py:504-523, 563-594, 661-664)."""
     B, H, S, D = 4, 4, 300, 64
     print(f"case compile_model mem_eff_attention lengths causal={causal} var_q={var_q}", flush=True)
@@ -232,11 +232,8 @@ def test_mem_eff_attention_variable_lengths(causal, var_q, copy_op):
         feed["lengths_q"] = lengths_q.cuda()
     y = torch.empty(B, S, H, D, dtype=torch.float16, device="cuda")
     module.run_with_tensors(feed, [y])
-    want = oracle.torch_mem_eff_attention(q, k, v, causal, lengths_kv).half().float()
-    got = y.cpu().float()
-    if var_q:
-        blank = (torch.arange(S)[None, :] >= lengths_q.long())[:, :, None, None]
-        got, want = got.masked_fill(blank, 0.0), want.masked_fill(blank, 0.0)
+    want = oracle.torch_mem_eff_attention(q, k, v, causal, lengths_kv, lengths_q if var_q else None).half().float()
+    got = y.cpu().float()   # (rows past a query length: zeros on both sides; the reference's test blanks them)
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
     module.close()
 

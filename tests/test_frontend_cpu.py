@@ -603,10 +603,10 @@ def test_mem_eff_attention_op_shapes_keys_and_hooks():
     y._attrs["name"] = "y"
     decl = registry.get("rocm.mem_eff_attention.func_decl")(op._attrs)
     assert decl.startswith("void mem_eff_attention_0(void* output, const void* q, const void* k, const void* v, "
-                           "const void* lengths_kv, int64_t* batch_size, int64_t* seq_len, int64_t* seq_len_kv, "
-                           "int num_heads, ")
+                           "const void* lengths_kv, const void* lengths_q, int64_t* batch_size, int64_t* seq_len, "
+                           "int64_t* seq_len_kv, int num_heads, ")
     call = registry.get("rocm.mem_eff_attention.func_call")(op._attrs)
-    assert call == (f"  mem_eff_attention_0(y, q, k, v, nullptr, &q_dim_0, &q_dim_2, &k_dim_2, 8, 40, 48, "
+    assert call == (f"  mem_eff_attention_0(y, q, k, v, nullptr, nullptr, &q_dim_0, &q_dim_2, &k_dim_2, 8, 40, 48, "
                     f"{40 ** -0.5!r}f, stream);")
     causal_op = ops.mem_eff_attention(causal=True)
     causal_op(q, k, v)
@@ -617,7 +617,7 @@ def test_mem_eff_attention_op_shapes_keys_and_hooks():
     assert ("aitamd_mem_eff_attention(0, q, k, v, output, *batch_size, num_heads, *seq_len, *seq_len_kv, head_dim,"
             in src)
     assert "head_dim_v, softmax_scale, 0," in src and "head_dim_v, softmax_scale, 1," in causal_src
-    # key lengths: a fourth (and, for query lengths, fifth) input of dtype "int"; only the key lengths reach the kernel
+    # key lengths: a fourth (and, for query lengths, fifth) input of dtype "int"
     var = ops.mem_eff_attention(causal=False, variable_seq_length_kv=True, variable_seq_length_q=True)
     lens_kv = Tensor([2, 1], name="lens_kv", dtype="int", is_input=True)
     lens_q = Tensor([2, 1], name="lens_q", dtype="int", is_input=True)
@@ -627,7 +627,12 @@ def test_mem_eff_attention_op_shapes_keys_and_hooks():
     var._attrs["name"] = "mem_eff_attention_2"
     y2._attrs["name"] = "y2"
     assert registry.get("rocm.mem_eff_attention.func_call")(var._attrs).startswith(
-        "  mem_eff_attention_2(y2, q, k, v, lens_kv, &q_dim_0,")
+        "  mem_eff_attention_2(y2, q, k, v, lens_kv, lens_q, &q_dim_0,")
+    only_q = ops.mem_eff_attention(causal=False, variable_seq_length_q=True)
+    y3 = only_q(q, k, v, None, lens_q)
+    only_q._attrs["name"], y3._attrs["name"] = "mem_eff_attention_3", "y3"
+    assert registry.get("rocm.mem_eff_attention.func_call")(only_q._attrs).startswith(
+        "  mem_eff_attention_3(y3, q, k, v, nullptr, lens_q, &q_dim_0,")
     copy = ops.mem_eff_attention(**var._get_op_attributes())
     assert copy._attrs["variable_seq_length_kv"] and copy._attrs["variable_seq_length_q"]
     with pytest.raises(AssertionError):

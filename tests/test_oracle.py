@@ -322,6 +322,13 @@ def test_mem_eff_attention_key_lengths(causal):
         mask = mask & torch.tril(torch.ones(S, Skv, dtype=torch.bool))
     sdpa = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask).permute(0, 2, 1, 3)
     assert torch.allclose(oracle.torch_mem_eff_attention(q, k, v, causal, lens), sdpa, atol=1e-5)
+    # query lengths only blank rows: everything before them is untouched
+    lq = torch.tensor([9, 3, 0], dtype=torch.int32)
+    with_q = oracle.torch_mem_eff_attention(q, k, v, causal, lens, lq)
+    base = oracle.torch_mem_eff_attention(q, k, v, causal, lens)
+    for b in range(batch):
+        assert torch.equal(with_q[b, :int(lq[b])], base[b, :int(lq[b])])
+        assert torch.count_nonzero(with_q[b, int(lq[b]):]) == 0
     # no keys at all: zeros by this library's convention
     zero = oracle.torch_mem_eff_attention(q, k, v, causal, torch.zeros(batch, 1, dtype=torch.int32))
     assert torch.count_nonzero(zero) == 0
