@@ -151,6 +151,10 @@ int attention_entry(const char* who, int dtype, const void* q, const void* k, co
   // grids of 128-row workgroups that leave CUs idle take the two-group form of those too: 8-19 % faster from 48 to
   // 256 workgroups (head dims 40 and 64), 7 % slower at 384
   if (mode == 0 && dma && groups_pay && ((M + 127) / 128) * B <= 256) mode = 3;
+  // head dim 64: the 256-row form with two wave groups when its grid is at most one workgroup per CU (and the
+  // 128-row grid is too large for the rule above): 5-10 % faster on 4 x 16384^2, 8 x 8192^2, 16 x 4096^2, 32 x 2048^2;
+  // no gain from 512 workgroups on
+  if (mode == 0 && dma && groups_pay && (16 * ks + 32 * ot) <= 128 && ((M + 255) / 256) * B <= 256) mode = 2;
   // AITAMD_ATTN_MODE=0|1|2|3 forces a variant where the shape allows it (a test and measurement knob)
   if (const char* forced = getenv("AITAMD_ATTN_MODE")) {
     const int m = atoi(forced);
