@@ -84,6 +84,7 @@ EXPORTED_SYMBOLS = [
     "aitamd_bmm_rcr",
     "aitamd_bmm_softmax_bmm_permute",
     "aitamd_mem_eff_attention",
+    "aitamd_attention_set_variant",
 ]
 
 _lock = threading.Lock()
@@ -145,6 +146,8 @@ def load() -> ctypes.CDLL:
         lib.aitamd_mem_eff_attention.restype = i32
         lib.aitamd_mem_eff_attention.argtypes = [i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, i32,
                                                  vp, vp, vp]
+        lib.aitamd_attention_set_variant.restype = i32
+        lib.aitamd_attention_set_variant.argtypes = [i32]
         _lib = lib
         return lib
 

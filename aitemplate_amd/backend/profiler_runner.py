@@ -73,10 +73,18 @@ class ProfilerRunner:
                 try:
                     out, err, rc = self._run_once(cmds, device)
                 except subprocess.TimeoutExpired:
-                    err, rc, out = f"timed out after {self._timeout}s", -1, ""
+                    out, err, rc = "", f"timed out after {self._timeout}s", None
                 result, failed = extract_profile_result(out, return_ops)
                 if not failed or rc == 0:
                     break
+                if rc is None or rc < 0:
+                    # The child hung or was ended by a signal (a GPU memory fault aborts it): running the
+                    # same command again would repeat that on the device.  Report it once, do not retry.
+                    how = "timed out" if rc is None else f"was killed by signal {-rc}"
+                    with self._lock:
+                        self._errors.append(
+                            f"Profiler {how} (not retried): {' '.join(map(str, cmds))}\n{err}")
+                    return
                 time.sleep(PROFILER_RUN_RETRY_DELAY_SECONDS)
             if failed and callback is None:
                 with self._lock:

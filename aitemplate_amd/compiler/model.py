@@ -103,29 +103,42 @@ def _reshape_tensor(tensor, shape: List[int]):
 
 class Model:
     class _DLLWrapper:
-        """Attribute access yields the C function wrapped with error checking; closed libraries raise."""
+        """The loaded model library.  Looking up an exported function returns a callable that raises when the
+        function reports a non-zero AITemplateError; once closed, every lookup raises."""
 
         def __init__(self, lib_path: str):
             self.lib_path = lib_path
             self.DLL = ctypes.cdll.LoadLibrary(lib_path)
             self.is_open = True
+            self._checked = {}
 
         def close(self):
-            if self.is_open:
-                _dlclose(self.DLL)
-                self.is_open = False
+            if not self.is_open:
+                return
+            self.is_open = False
+            self._checked.clear()
+            _dlclose(self.DLL)
+
+        def _make_checked(self, name: str):
+            c_func = getattr(self.DLL, name)
+
+            def call(*args):
+                if c_func(*args) != 0:
+                    raise RuntimeError(f"Error in function: {name}")
+
+            call.__name__ = name
+            return call
 
         def __getattr__(self, name):
-            if not self.is_open:
-                raise RuntimeError(f"Cannot use closed AIT library: {self.lib_path}")
-            method = getattr(self.DLL, name)
-
-            def _wrapped_func(*args):
-                err = method(*args)
-                if err:
-                    raise RuntimeError(f"Error in function: {method.__name__}")
-
-            return _wrapped_func
+            # only reached for names that are not instance attributes, i.e. the library's symbols
+            if name.startswith("__") or not self.__dict__.get("is_open", False):
+                if name.startswith("__"):
+                    raise AttributeError(name)
+                raise RuntimeError(f"Cannot use closed AIT library: {self.__dict__.get('lib_path')}")
+            fn = self._checked.get(name)
+            if fn is None:
+                fn = self._checked[name] = self._make_checked(name)
+            return fn
 
     def __init__(self, lib_path: str, num_runtimes: int = 1,
                  allocator_kind: Optional[AITemplateAllocatorKind] = None):

@@ -1,4 +1,5 @@
 // C ABI launcher of the fused attention kernel (bmm_softmax_bmm_permute).
+#include <atomic>
 #include <cstdlib>
 #include <mutex>
 
@@ -10,6 +11,21 @@ namespace aitamd {
 namespace {
 
 constexpr int kMaxDevices = 64;
+
+// Variant forced by aitamd_attention_set_variant: -1 automatic, 0..3 a MODE below.  The environment variable
+// AITAMD_ATTN_MODE gives the initial value and is read once, not on every launch.
+constexpr int kVariantUnset = -2;
+std::atomic<int> g_forced_variant{kVariantUnset};
+int forced_variant() {
+  int m = g_forced_variant.load(std::memory_order_relaxed);
+  if (m == kVariantUnset) {
+    const char* env = getenv("AITAMD_ATTN_MODE");
+    const int from_env = env ? atoi(env) : -1;
+    g_forced_variant.compare_exchange_strong(m, from_env >= 0 && from_env <= 3 ? from_env : -1);
+    m = g_forced_variant.load(std::memory_order_relaxed);
+  }
+  return m;
+}
 
 // MODE 0: four waves (128 query rows), two LDS stages, two workgroups per CU.
 // MODE 1: eight waves (256 query rows) share each K / V tile and four LDS stages keep three tiles in flight.
@@ -59,7 +75,9 @@ hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  hipError_t attr_err = hipSuccess;
+  // the outcome is kept per device: a failed opt-in must fail every later call too, not only the first
+  static hipError_t attr_errs[kMaxDevices];
+  hipError_t& attr_err = attr_errs[dev % kMaxDevices];
   std::call_once(once[dev % kMaxDevices], [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);
@@ -155,9 +173,9 @@ int attention_entry(const char* who, int dtype, const void* q, const void* k, co
   // 128-row grid is too large for the rule above): 5-10 % faster on 4 x 16384^2, 8 x 8192^2, 16 x 4096^2, 32 x 2048^2;
   // no gain from 512 workgroups on
   if (mode == 0 && dma && groups_pay && (16 * ks + 32 * ot) <= 128 && ((M + 255) / 256) * B <= 256) mode = 2;
-  // AITAMD_ATTN_MODE=0|1|2|3 forces a variant where the shape allows it (a test and measurement knob)
-  if (const char* forced = getenv("AITAMD_ATTN_MODE")) {
-    const int m = atoi(forced);
+  // aitamd_attention_set_variant(0|1|2|3) forces a variant where the shape allows it (a test and measurement knob)
+  {
+    const int m = forced_variant();
     if (m >= 0 && m <= 2 && dma && (16 * ks + 32 * ot) <= 128) mode = m;
     if (m == 3 && dma) mode = 3;
   }
@@ -181,6 +199,12 @@ int attention_entry(const char* who, int dtype, const void* q, const void* k, co
 }
 
 }  // namespace
+
+extern "C" int aitamd_attention_set_variant(int variant) {
+  if (variant < -1 || variant > 3) return fail("aitamd_attention_set_variant: variant %d is not one of -1, 0, 1, 2, 3", variant);
+  g_forced_variant.store(variant, std::memory_order_relaxed);
+  return 0;
+}
 
 extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const void* k, const void* v, void* out,
                                               int64_t B, int64_t M, int64_t N, int64_t K, int64_t O, int64_t G,

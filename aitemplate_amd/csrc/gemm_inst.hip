@@ -98,7 +98,9 @@ hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  hipError_t attr_err = hipSuccess;
+  // the outcome is kept per device: a failed opt-in must fail every later call too, not only the first
+  static hipError_t attr_errs[kMaxDevices];
+  hipError_t& attr_err = attr_errs[dev % kMaxDevices];
   std::call_once(once[dev % kMaxDevices], [&] {
     attr_err = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Tile::kLdsBytes);

@@ -69,10 +69,14 @@ def gemm(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor]
         raise ValueError(f"b must be [N, K={K}], got {tuple(b.shape)}")
     if out is None:
         out = torch.empty(*lead, N, dtype=dtype, device=a.device)
-    out2 = out.reshape(M, N)
+    if out.dim() == 2 and out.shape == (M, N) and out.stride(1) == 1 and out.stride(0) >= N:
+        out2 = out  # a row-pitched view (rows of a wider buffer) is written in place with ldc = its pitch
+    else:
+        _check_out(out, M * N, "M*N")
+        out2 = out.view(M, N)
     nres = _kernels.NUM_RESIDUALS_OF_EPILOGUE[epi]
-    if epi != 0 and (bias is None or bias.numel() != N):
-        raise ValueError("bias must be 1-D of size N")
+    if epi != 0 and (bias is None or bias.numel() != N or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous 1-D tensor of size N")
     d0_2 = d0.reshape(M, N) if d0 is not None else None
     d1_2 = d1.reshape(M, N) if d1 is not None else None
     if nres >= 1 and (d0_2 is None or d0_2.shape != out2.shape):
@@ -87,6 +91,14 @@ def gemm(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor]
                              ldd, _stream_ptr())
     _kernels.check(rc, op)
     return out
+
+
+def _check_out(out: torch.Tensor, numel: int, what: str) -> None:
+    """A caller's output buffer is written in place through its raw pointer: it has to be dense and of the
+    result's size, or the kernel would write past it (or into a temporary copy)."""
+    if not out.is_contiguous() or out.numel() != numel:
+        raise ValueError(f"out must be contiguous with {what} = {numel} elements, got shape {tuple(out.shape)} "
+                         f"strides {tuple(out.stride())}")
 
 
 def gemm_permute(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor], shape,
@@ -110,8 +122,8 @@ def gemm_permute(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch
     if b.dim() != 2 or b.shape[b_k] != K:
         raise ValueError(f"b does not match K={K}: got {tuple(b.shape)}")
     M, N = a2.shape[0], b.shape[b_n]
-    if epi != 0 and (bias is None or bias.numel() != N):
-        raise ValueError("bias must be 1-D of size N")
+    if epi != 0 and (bias is None or bias.numel() != N or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous 1-D tensor of size N")
     t1, t2, t3 = (int(t) for t in shape)
     if layout == _kernels.PERMUTE_M2N3:
         if M % t1 or N % (t2 * t3):
@@ -151,6 +163,8 @@ def bmm_rcr(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None
         raise ValueError("K mismatch")
     if out is None:
         out = torch.empty(B, M, N, dtype=dtype, device=a.device)
+    else:
+        _check_out(out, B * M * N, "B*M*N")
     sa = 0 if (a3.shape[0] == 1 and B > 1) else M * K
     sb = 0 if (b3.shape[0] == 1 and B > 1) else N * K
     rc = lib.aitamd_bmm_rcr(_TORCH_DTYPE_ID[dtype], algo, _p(a3), _p(b3), _p(out), B, M, N, K, K, K, N, sa, sb,
@@ -215,6 +229,8 @@ def bmm_add(layout: str, a: torch.Tensor, b: torch.Tensor, d0: torch.Tensor, out
         raise ValueError(f"d0 must be [{B}, {M}, {N}], got {tuple(d0.shape)}")
     if out is None:
         out = torch.empty(B, M, N, dtype=dtype, device=a.device)
+    else:
+        _check_out(out, B * M * N, "B*M*N")
     rc = lib.aitamd_bmm_add(lay, _TORCH_DTYPE_ID[dtype], algo, _p(a), _p(b), _p(d0), _p(out), B, M, N, K, a.shape[2],
                             b.shape[2], N, N, M * K, N * K, M * N, M * N, _stream_ptr())
     _kernels.check(rc, f"bmm_{layout}_add")
@@ -275,6 +291,8 @@ def bmm_softmax_bmm_permute(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, s
     G = int(shape[0])
     if out is None:
         out = torch.empty(B // G, M, G, O, dtype=dtype, device=q.device)
+    else:
+        _check_out(out, B * M * O, "B*M*O")
     rc = lib.aitamd_bmm_softmax_bmm_permute(_TORCH_DTYPE_ID[dtype], _p(q), _p(k), _p(v), _p(out), B, M, N, K, O, G,
                                             float(scale), int(bool(causal)), _stream_ptr())
     _kernels.check(rc, "bmm_softmax_bmm_permute")
@@ -306,6 +324,8 @@ def mem_eff_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal:
             raise ValueError(f"{name} must be a contiguous int32 tensor with one entry per batch on the operands' device")
     if out is None:
         out = torch.empty(batch, seq_q, heads, head_dim_v, dtype=dtype, device=q.device)
+    else:
+        _check_out(out, batch * seq_q * heads * head_dim_v, "batch*seq_q*heads*head_dim_v")
     rc = lib.aitamd_mem_eff_attention(_TORCH_DTYPE_ID[dtype], _p(q), _p(k), _p(v), _p(out), batch, heads, seq_q, seq_kv,
                                       head_dim, head_dim_v, float(head_dim) ** -0.5, int(bool(causal)),
                                       _p(lengths_kv), _p(lengths_q), _stream_ptr())

@@ -56,6 +56,11 @@ std::vector<uint64_t> ModelBase::CurrentSignature() const {
     sig.push_back(reinterpret_cast<uint64_t>(p.ptr));
     for (const auto& d : p.shape_ptrs) sig.push_back(static_cast<uint64_t>(*d.value));
   }
+  // Unbound constants are bound through members of the generated class, not through params_, and the bound
+  // ones through the blob base: a captured graph holds their addresses, so both belong to the signature.
+  // (The map is not modified after construction, so its iteration order is the same on every call.)
+  for (const auto& kv : constant_name_to_ptr_) sig.push_back(reinterpret_cast<uint64_t>(*kv.second));
+  sig.push_back(reinterpret_cast<uint64_t>(constants_));
   return sig;
 }
 

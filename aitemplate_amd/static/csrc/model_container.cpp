@@ -53,9 +53,10 @@ ModelContainer::~ModelContainer() {
     pending_.clear();
   }
   models_.clear();
-  if (constants_blob_ != nullptr) {
+  for (uint8_t* blob : {constants_blob_, staged_blob_}) {
+    if (blob == nullptr) continue;
     try {
-      allocator_.Free(constants_blob_);
+      allocator_.Free(blob);
     } catch (...) {
     }
   }
@@ -342,14 +343,38 @@ void ModelContainer::SetConstant(const char* name, const AITData& tensor, bool u
   if (tensor.ptr == nullptr && c.num_bytes != 0) throw std::runtime_error(std::string("Null data for constant ") + name);
   std::unique_lock<std::shared_mutex> lk(constants_mutex_);
   if (c.bound) {
-    // a constant with embedded bytes is overwritten in place (device-to-device copy)
-    if (c.num_bytes > 0) {
-      AIT_DEVICE_CHECK(hipMemcpyAsync(constants_blob_ + c.offset, tensor.ptr, c.num_bytes, hipMemcpyDeviceToDevice, stream));
-      AIT_DEVICE_CHECK(hipStreamSynchronize(stream));
+    if (c.num_bytes == 0) return;
+    // Run() gives up the shared lock once its kernels are queued, so a runtime may still be reading the
+    // blob on another stream: drain every runtime before bytes change (reference:
+    // static/csrc/model_container.cpp:452-455, WaitForAllModels before any SetConstant).
+    WaitForAllModels();
+    uint8_t* dst = constants_blob_;
+    if (use_inactive_set) {
+      // double buffering: the bytes go to a second blob that SwapConstants() makes the active one
+      // (reference: static/csrc/model_container.cpp:661-680).  The first staged write after a swap starts
+      // from a copy of the active blob, so constants that are not staged keep their current values.
+      if (staged_blob_ == nullptr) staged_blob_ = static_cast<uint8_t*>(allocator_.Allocate(meta_->constants_size));
+      if (!staged_blob_in_use_) {
+        AIT_DEVICE_CHECK(hipMemcpyAsync(staged_blob_, constants_blob_, meta_->constants_size, hipMemcpyDeviceToDevice, stream));
+        staged_blob_in_use_ = true;
+      }
+      dst = staged_blob_;
     }
+    AIT_DEVICE_CHECK(hipMemcpyAsync(dst + c.offset, tensor.ptr, c.num_bytes, hipMemcpyDeviceToDevice, stream));
+    AIT_DEVICE_CHECK(hipStreamSynchronize(stream));
     return;
   }
   unbound_ptrs_[use_inactive_set ? 1 : 0][c.name] = tensor.ptr;
+}
+
+// Caller holds constants_mutex_ exclusively, so no Run() can start meanwhile.
+void ModelContainer::WaitForAllModels() {
+  std::unique_lock<std::mutex> lk(pool_mutex_);
+  for (ModelBase* m : pending_) {
+    m->WaitForCompletion();
+    available_.push_back(m);
+  }
+  pending_.clear();
 }
 
 size_t ModelContainer::GetNumConstants(bool unbound_only, bool folding_inputs_only) const {
@@ -382,6 +407,13 @@ void ModelContainer::SwapConstants() {
   std::unique_lock<std::shared_mutex> lk(constants_mutex_);
   // entries staged in the inactive set replace the active ones; unstaged names keep their binding
   for (auto& kv : unbound_ptrs_[1]) std::swap(unbound_ptrs_[0][kv.first], kv.second);
+  if (staged_blob_in_use_) {
+    // the staged blob becomes the one every runtime reads; the old one is the next staging area
+    WaitForAllModels();
+    std::swap(constants_blob_, staged_blob_);
+    staged_blob_in_use_ = false;
+    for (auto& m : models_) m->SetConstantsBlob(constants_blob_);
+  }
 }
 
 // ---- metadata ---------------------------------------------------------------

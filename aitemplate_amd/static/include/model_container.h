@@ -72,12 +72,15 @@ class ModelContainer {
   void ReturnModel(ModelBase* m, bool failed);
   void PrepareForRun(ModelBase* m, const AITData* inputs, size_t num_inputs, AITData* outputs, size_t num_outputs);
   const ConstantMeta& FindConstant(const char* name) const;
+  void WaitForAllModels();
   float BenchmarkImpl(const AITData* inputs, size_t num_inputs, AITData* outputs, size_t num_outputs,
                       StreamType stream, bool graph_mode, size_t count, int64_t** output_shapes_out);
 
   const ModelMeta* meta_;
   AITemplateAllocator& allocator_;
-  uint8_t* constants_blob_ = nullptr;  // device image of the bound constants
+  uint8_t* constants_blob_ = nullptr;  // device image of the bound constants (the one the runtimes read)
+  uint8_t* staged_blob_ = nullptr;     // second image: takes double-buffered updates until SwapConstants()
+  bool staged_blob_in_use_ = false;    // staged_blob_ holds updates that have not been swapped in yet
   std::vector<std::unique_ptr<ModelBase>> models_;
   std::vector<ModelBase*> available_;
   std::vector<ModelBase*> pending_;

@@ -217,6 +217,14 @@ AITAMD_API int aitamd_mem_eff_attention(int dtype,
                                         int64_t head_dim, int64_t head_dim_v, float scale, int causal,
                                         const int32_t* lengths_kv, const int32_t* lengths_q, void* stream);
 
+/* Test and measurement knob of the two attention entry points above: force one of the kernel's four work
+ * decompositions wherever the shape allows it (0: four waves per 128 query rows; 1: eight waves per 256 rows;
+ * 2: as 1 with two wave groups on alternate key tiles; 3: as 0 with two wave groups), or -1 (the default) to let
+ * the launcher choose from the shape.  Process-wide; the results are the same in every variant up to rounding.
+ * The environment variable AITAMD_ATTN_MODE sets the initial value and is read once.  No counterpart in the
+ * reference (CK instances are chosen by its profiler only). */
+AITAMD_API int aitamd_attention_set_variant(int variant);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -28,3 +28,17 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def attn_variant():
+    """Force one of the attention kernel's work decompositions for a test; automatic choice again afterwards."""
+    from aitemplate_amd import _kernels
+
+    lib = _kernels.load()
+
+    def force(variant):
+        _kernels.check(lib.aitamd_attention_set_variant(int(variant)), "aitamd_attention_set_variant")
+
+    yield force
+    lib.aitamd_attention_set_variant(-1)

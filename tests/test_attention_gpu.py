@@ -64,10 +64,10 @@ def test_ragged_and_odd_shapes(B, M, N, K, O, G, causal):
     (2, 40, 50, 40, 40, 2, True, None),        # a single tile: the second group has nothing to merge
     (2, 260, 0, 40, 40, 2, False, None),       # no keys at all
 ])
-def test_every_variant_of_the_small_head_dims(monkeypatch, mode, B, M, N, K, O, G, causal, scale):
-    # AITAMD_ATTN_MODE picks the variant where the shape allows it: 0 four waves, 1 eight waves, 2 (3) two groups of
+def test_every_variant_of_the_small_head_dims(attn_variant, mode, B, M, N, K, O, G, causal, scale):
+    # aitamd_attention_set_variant picks the variant where the shape allows it: 0 four waves, 1 eight waves, 2 (3) two groups of
     # eight (four) waves that take alternate key tiles and merge their running sums at the end
-    monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+    attn_variant(mode)
     print(f"case attention mode={mode} B={B} M={M} N={N} K={K} causal={causal} scale={scale}", flush=True)
     _check(B, M, N, K, O, G, causal=causal, scale=scale, seed=mode + N)
 
@@ -153,10 +153,10 @@ def _check_mem_eff(batch, heads, S, Skv, d, dv, lens, causal=False, dtype=torch.
     (2, 2, 40, 50, 40, 40, [50, 49], False),                 # single tile
     (2, 3, 64, 200, 64, 128, [1200, -3], False),             # lengths are clamped to [0, Skv]
 ])
-def test_mem_eff_attention_key_lengths(monkeypatch, mode, batch, heads, S, Skv, d, dv, lens, causal):
+def test_mem_eff_attention_key_lengths(attn_variant, mode, batch, heads, S, Skv, d, dv, lens, causal):
     """Key lengths through the C ABI for every kernel variant (as in test_attention.py:504-523 of the reference)."""
     if mode is not None:
-        monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+        attn_variant(mode)
     _check_mem_eff(batch, heads, S, Skv, d, dv, lens, causal=causal, seed=Skv)
 
 
@@ -173,10 +173,10 @@ def test_mem_eff_attention_shapes_and_dtypes(dtype, batch, heads, S, Skv, d, dv,
 
 @pytest.mark.parametrize("mode", [None, 0, 1, 2, 3])
 @pytest.mark.parametrize("causal", [False, True])
-def test_mem_eff_attention_query_lengths(monkeypatch, mode, causal):
+def test_mem_eff_attention_query_lengths(attn_variant, mode, causal):
     """Rows past a query length are zeros (whole blocks of them visit no keys), the rows before are unchanged."""
     if mode is not None:
-        monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+        attn_variant(mode)
     _check_mem_eff(5, 2, 700, 640, 40, 40, [640, 300, 640, 1, 640], causal=causal, seed=mode or 9,
                    lens_q=[700, 130, 0, 257, 9000])
 

@@ -276,6 +276,42 @@ def test_profiler_runner_parses_output_and_picks_fastest(tmp_path):
         bad.join()
 
 
+def test_profiler_runner_does_not_rerun_a_killed_or_hung_profiler(tmp_path):
+    """A profiler ended by a signal (what a GPU fault does to it) or by the time limit ran once only."""
+    from aitemplate_amd.compiler.ops.gemm_universal.gemm_common import GemmProfilerPostprocessingDelegate
+
+    log = tmp_path / "runs.log"
+    killed = tmp_path / "killed.sh"
+    killed.write_text(f"#!/bin/sh\necho ran >> {log}\nkill -ABRT $$\n")
+    killed.chmod(killed.stat().st_mode | stat.S_IEXEC)
+    pr = ProfilerRunner(devices=["0"], postprocessing_delegate=GemmProfilerPostprocessingDelegate(), timeout=30)
+    pr.push([str(killed)], process_result_callback=None, return_ops=["x"])
+    with pytest.raises(RuntimeError, match="killed by signal 6"):
+        pr.join()
+    assert log.read_text().count("ran") == 1
+
+    log.write_text("")
+    hung = tmp_path / "hung.sh"
+    hung.write_text(f"#!/bin/sh\necho ran >> {log}\nexec sleep 20\n")
+    hung.chmod(hung.stat().st_mode | stat.S_IEXEC)
+    pr = ProfilerRunner(devices=["0"], postprocessing_delegate=GemmProfilerPostprocessingDelegate(), timeout=1)
+    pr.push([str(hung)], process_result_callback=None, return_ops=["x"])
+    with pytest.raises(RuntimeError, match="timed out"):
+        pr.join()
+    assert log.read_text().count("ran") == 1
+
+    # an ordinary failure (exit status above 0, nothing printed) is still tried again
+    log.write_text("")
+    flaky = tmp_path / "flaky.sh"
+    flaky.write_text(f"#!/bin/sh\necho ran >> {log}\nexit 3\n")
+    flaky.chmod(flaky.stat().st_mode | stat.S_IEXEC)
+    pr = ProfilerRunner(devices=["0"], postprocessing_delegate=GemmProfilerPostprocessingDelegate(), timeout=30)
+    pr.push([str(flaky)], process_result_callback=None, return_ops=["x"])
+    with pytest.raises(RuntimeError, match="Profiler failure"):
+        pr.join()
+    assert log.read_text().count("ran") == 3
+
+
 # ---- passes and code generation ----------------------------------------------------------------
 def test_naming_aliases_and_memory_planning():
     reset_name_counters()

@@ -236,6 +236,64 @@ def test_unbound_and_bound_constants():
     mod.close()
 
 
+def test_graph_mode_sees_new_constants():
+    """A replayed graph must not keep the weight addresses it was captured with."""
+    x, w, b, want = _data(16)
+    y = torch.empty(16, N, dtype=torch.float16, device="cuda")
+    want2 = oracle.torch_gemm("gemm_rcr_bias", x, w * 2, b).half().float()
+    # unbound constants: a new buffer through SetConstant, then through the double buffer + swap
+    mod = compile_model(_graph(weight_as_constant=True), detect_target(), WORKDIR, "model_api_unbound_graph")
+    wc, bc, w2 = w.cuda(), b.cuda(), (w * 2).cuda()
+    mod.set_many_constants_with_tensors({"weight": wc, "bias": bc})
+    for _ in range(2):
+        mod.run_with_tensors([x.cuda()], [y], graph_mode=True)
+        torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    mod.set_constant_with_tensor("weight", w2)
+    for _ in range(2):
+        mod.run_with_tensors([x.cuda()], [y], graph_mode=True)
+        torch.testing.assert_close(y.cpu().float(), want2, atol=2e-2, rtol=1e-2)
+    mod.set_double_buffer_constant_with_tensor("weight", wc)
+    mod.run_with_tensors([x.cuda()], [y], graph_mode=True)
+    torch.testing.assert_close(y.cpu().float(), want2, atol=2e-2, rtol=1e-2)
+    mod.swap_constants()
+    mod.run_with_tensors([x.cuda()], [y], graph_mode=True)
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    mod.close()
+
+
+def test_bound_constant_double_buffer_takes_effect_at_the_swap():
+    x, w, b, want = _data(16)
+    y = torch.empty(16, N, dtype=torch.float16, device="cuda")
+    want2 = oracle.torch_gemm("gemm_rcr_bias", x, w * 2, b).half().float()
+    want3 = oracle.torch_gemm("gemm_rcr_bias", x, w * 2, b * 3).half().float()
+    mod = compile_model(_graph(weight_as_constant=True), detect_target(), WORKDIR, "model_api_bound_swap",
+                        constants={"weight": w, "bias": b})
+    for graph_mode in (False, True):
+        mod.run_with_tensors([x.cuda()], [y], graph_mode=graph_mode)
+        torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    mod.set_double_buffer_constant_with_tensor("weight", (w * 2).cuda())
+    for graph_mode in (False, True):  # staged only: the active weights are the compiled-in ones
+        mod.run_with_tensors([x.cuda()], [y], graph_mode=graph_mode)
+        torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    mod.swap_constants()
+    for graph_mode in (False, True):  # the bias was not staged and keeps its value
+        mod.run_with_tensors([x.cuda()], [y], graph_mode=graph_mode)
+        torch.testing.assert_close(y.cpu().float(), want2, atol=2e-2, rtol=1e-2)
+    # a second round: the blob that was active first is the staging area now
+    mod.set_many_double_buffer_constants_with_tensors({"bias": (b * 3).cuda()})
+    mod.run_with_tensors([x.cuda()], [y])
+    torch.testing.assert_close(y.cpu().float(), want2, atol=2e-2, rtol=1e-2)
+    mod.swap_constants()
+    for graph_mode in (True, False):
+        mod.run_with_tensors([x.cuda()], [y], graph_mode=graph_mode)
+        torch.testing.assert_close(y.cpu().float(), want3, atol=2e-2, rtol=1e-2)
+    # the direct call writes the active blob at once
+    mod.set_constant_with_tensor("bias", b.cuda())
+    mod.run_with_tensors([x.cuda()], [y], graph_mode=True)
+    torch.testing.assert_close(y.cpu().float(), want2, atol=2e-2, rtol=1e-2)
+    mod.close()
+
+
 def test_ait_recompile_0_loads_existing_library(module, monkeypatch):
     monkeypatch.setenv("AIT_RECOMPILE", "0")
     mod = compile_model(_graph(), detect_target(), WORKDIR, "model_api_simple")

@@ -75,7 +75,7 @@ def test_bmm_layouts_random_shapes():
         assert ok, f"case {i} bmm_{layout} B={B} M={M} N={N} K={K} {dtype} add={add}: max error {err}"
 
 
-def test_attention_random_shapes(monkeypatch):
+def test_attention_random_shapes(attn_variant):
     rng = random.Random(1234)
     for i in range(150):
         G = rng.choice([1, 2, 4, 8])
@@ -89,9 +89,9 @@ def test_attention_random_shapes(monkeypatch):
         scale = rng.choice([K ** -0.5, K ** -0.5, 0.3, -0.2, 1.0 / 8])
         mode = rng.choice([None, 0, 1, 2, 3])  # kernel variant, where the head dims allow the choice
         if mode is None:
-            monkeypatch.delenv("AITAMD_ATTN_MODE", raising=False)
+            attn_variant(-1)
         else:
-            monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+            attn_variant(mode)
         g = torch.Generator().manual_seed(i)
         q = torch.randn(B, M, K, generator=g).to(dtype)
         k = torch.randn(B, N, K, generator=g).to(dtype)
@@ -105,7 +105,7 @@ def test_attention_random_shapes(monkeypatch):
         assert ok, f"case {i}: max error {err}"
 
 
-def test_mem_eff_attention_random_shapes_and_key_lengths(monkeypatch):
+def test_mem_eff_attention_random_shapes_and_key_lengths(attn_variant):
     rng = random.Random(4321)
     for i in range(100):
         heads = rng.choice([1, 2, 4, 8])
@@ -118,9 +118,9 @@ def test_mem_eff_attention_random_shapes_and_key_lengths(monkeypatch):
         dtype = torch.float16 if rng.random() < 0.7 else torch.bfloat16
         mode = rng.choice([None, 0, 1, 2, 3])
         if mode is None:
-            monkeypatch.delenv("AITAMD_ATTN_MODE", raising=False)
+            attn_variant(-1)
         else:
-            monkeypatch.setenv("AITAMD_ATTN_MODE", str(mode))
+            attn_variant(mode)
         lens = None
         if rng.random() < 0.8:
             lens = torch.tensor([rng.choice([0, 1, Skv, Skv // 2, rng.randint(0, Skv)]) for _ in range(batch)],
