@@ -23,6 +23,10 @@
 
 #include "gemm_kernel_dma.hpp"
 
+#ifndef TILE_STAMP
+#define TILE_STAMP(i, k)
+#endif
+
 namespace aitamd {
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_>
@@ -224,7 +228,96 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   const int r_row = lane / SC;
   const int r_c = lane % SC;
 
+  // Fast form of the epilogue's addressing (plain store, everything 16-byte aligned, a tile's rows span less than
+  // 2 GiB): the output and the residuals are addressed through buffer descriptors that start at the wave's
+  // corner of the tile, with 32-bit byte offsets that advance by a scalar per 8-row pass - no 64-bit index
+  // arithmetic per pass, rows past M cut off by the descriptor's size, columns past N by an out-of-range offset.
+  const bool fast_addr = !PERM && vec_ok && (int64_t)BM * p.ldc * 2 < 0x7fffffffll &&
+      (Epi::kNumD == 0 || (int64_t)BM * p.ldd * 2 < 0x7fffffffll);
+  const uint32_t lane_off_c = (uint32_t)((r_row * (int)p.ldc + r_c * 8) * 2);
+  const uint32_t lane_off_d = (uint32_t)((r_row * (int)p.ldd + r_c * 8) * 2);
+  auto uniform_ptr = [](const void* ptr) {
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+  };
+
+  auto epilogue_fast = [&](const TileCoord& c) {
+    const int m_w = c.m0 + wm * Tile::WTM;  // first row and column of the wave's part of the tile
+    const int n_w = c.n0 + wn * Tile::WTN;
+    const int rows_left = p.M - m_w;
+    const uint32_t rows_valid = rows_left <= 0 ? 0u : (uint32_t)(rows_left < Tile::WTM ? rows_left : Tile::WTM);
+    T* Cw = reinterpret_cast<T*>(p.c) + out_batch_offset(p, c.batch) + (int64_t)m_w * p.ldc + n_w;
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(uniform_ptr(Cw), rows_valid * (uint32_t)p.ldc * 2u);
+    __amdgpu_buffer_rsrc_t rd0 = rc, rd1 = rc;
+    if constexpr (Epi::kNumD >= 1) {
+      const T* Dw = reinterpret_cast<const T*>(p.d0) + (int64_t)c.batch * p.sd + (int64_t)m_w * p.ldd + n_w;
+      rd0 = make_rsrc(uniform_ptr(Dw), rows_valid * (uint32_t)p.ldd * 2u);
+    }
+    if constexpr (Epi::kNumD >= 2) {
+      const T* Dw = reinterpret_cast<const T*>(p.d1) + (int64_t)c.batch * p.sd + (int64_t)m_w * p.ldd + n_w;
+      rd1 = make_rsrc(uniform_ptr(Dw), rows_valid * (uint32_t)p.ldd * 2u);
+    }
+    const int n = n_w + r_c * 8;  // the lane's 8 columns: the same in every pass
+    const bool col_ok = n < p.N;
+    const uint32_t off_c0 = col_ok ? lane_off_c : kOobOffset;
+    const uint32_t off_d0 = col_ok ? lane_off_d : kOobOffset;
+    float bf8[8] = {};
+    if constexpr (Epi::kHasBias) {
+      if (col_ok) {
+        const vec8 bv = *reinterpret_cast<const vec8*>(bias + n);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) bf8[j] = Tr::to_float(bv[j]);
+      }
+    }
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          typename Tr::vec4 h;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) h[j] = Tr::from_float(acc[mi][ni][gq * 4 + j]);
+          *reinterpret_cast<u32x2*>(strip + w_base + (((ni * 4 + gq) ^ w_swz) << 4)) = __builtin_bit_cast(u32x2, h);
+        }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      vec8 raw[Tile::PASSES], d0v[Tile::PASSES], d1v[Tile::PASSES];
+#pragma unroll
+      for (int ps = 0; ps < Tile::PASSES; ++ps) {
+        const int row = ps * Tile::ROWS_PER_PASS + r_row;
+        raw[ps] = *reinterpret_cast<const vec8*>(strip + row * Tile::STRIP_PITCH + ((r_c ^ (row & (SC - 1))) << 4));
+        const uint32_t step_d = (uint32_t)((mi * MT + ps * Tile::ROWS_PER_PASS) * (int)p.ldd * 2);
+        if constexpr (Epi::kNumD >= 1) d0v[ps] = __builtin_bit_cast(vec8, buffer_load_16B(rd0, off_d0 + step_d));
+        if constexpr (Epi::kNumD >= 2) d1v[ps] = __builtin_bit_cast(vec8, buffer_load_16B(rd1, off_d0 + step_d));
+      }
+#pragma unroll
+      for (int ps = 0; ps < Tile::PASSES; ++ps) {
+        vec8 o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          o[j] = Tr::from_float(Epi::apply(Tr::to_float(raw[ps][j]), bf8[j],
+                                           Epi::kNumD >= 1 ? Tr::to_float(d0v[ps][j]) : 0.f,
+                                           Epi::kNumD >= 2 ? Tr::to_float(d1v[ps][j]) : 0.f));
+        const uint32_t off = off_c0 + (uint32_t)((mi * MT + ps * Tile::ROWS_PER_PASS) * (int)p.ldc * 2);
+        if (p.nt_store)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, 2);
+        else
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, 0);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  };
+
   auto epilogue = [&](const TileCoord& c) {
+    if (fast_addr) {
+      epilogue_fast(c);
+      return;
+    }
     T* Cb = reinterpret_cast<T*>(p.c) + out_batch_offset(p, c.batch);
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cb, kStoreRecords);
     const T* D0b = Epi::kNumD >= 1 ? reinterpret_cast<const T*>(p.d0) + (int64_t)c.batch * p.sd : nullptr;
@@ -305,6 +398,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     // waves whose rows lie outside a half tile keep the ring turning (their share of the loads, the
     // waits and the barriers) but multiply and store nothing; a half tile is always the last item
     const bool active = wm * Tile::WTM < cur.rows;
+    TILE_STAMP(i, 0);
     for (int kt = 0; kt < k_tiles; ++kt) {
       const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
       const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
@@ -335,7 +429,9 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       }
       rd_stage = nx_stage;
     }
+    TILE_STAMP(i, 1);
     if (active) epilogue(cur);
+    TILE_STAMP(i, 2);
   }
   // no LDS-DMA may be in flight into a workgroup that has ended
   wait_vmcnt<0>();
