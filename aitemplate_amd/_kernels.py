@@ -85,6 +85,8 @@ EXPORTED_SYMBOLS = [
     "aitamd_bmm_softmax_bmm_permute",
     "aitamd_mem_eff_attention",
     "aitamd_attention_set_variant",
+    "aitamd_gemm_workspace_bytes",
+    "aitamd_gemm_rcr_ws",
 ]
 
 _lock = threading.Lock()
@@ -146,6 +148,10 @@ def load() -> ctypes.CDLL:
         lib.aitamd_mem_eff_attention.restype = i32
         lib.aitamd_mem_eff_attention.argtypes = [i32, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, i32,
                                                  vp, vp, vp]
+        lib.aitamd_gemm_workspace_bytes.restype = i64
+        lib.aitamd_gemm_workspace_bytes.argtypes = [i32, i32, i32, i64, i64, i64, i64]
+        lib.aitamd_gemm_rcr_ws.restype = i32
+        lib.aitamd_gemm_rcr_ws.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp, i64, vp]
         lib.aitamd_attention_set_variant.restype = i32
         lib.aitamd_attention_set_variant.argtypes = [i32]
         _lib = lib

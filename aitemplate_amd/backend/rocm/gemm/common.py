@@ -188,14 +188,25 @@ namespace ait {
 FOOTER = "\n}  // namespace ait\n"
 
 
-def gemm_signature(func_name: str, op_name: str, a_rank: int, b_rank: int, c_rank: int, pdims: int = 0) -> str:
+def gemm_signature(func_name: str, op_name: str, a_rank: int, b_rank: int, c_rank: int, pdims: int = 0,
+                   with_workspace: bool = False) -> str:
     """Launcher prototype; `pdims` trailing `const int p_dim<i>` carry a permuting op's shape attribute
-    (reference: backend/rocm/gemm/common.py:140-160)."""
+    (reference: backend/rocm/gemm/common.py:140-160).  Ops whose profiled instance needs scratch memory take the
+    model's shared workspace and its size after the tensor pointers (the reference's CUDA launchers do the same,
+    backend/cuda/gemm_universal/common.py:317-345)."""
     ptrs = ["void* in_ptr", "void* weight_ptr", "void* out_ptr"] + [f"void* {p}" for p in extra_pointer_names(op_name)]
+    if with_workspace:
+        ptrs += ["uint8_t* workspace", "int64_t workspace_bytes"]
     dims = [f"int64_t* {n}" for n in dim_param_names("a", a_rank) + dim_param_names("b", b_rank)
             + dim_param_names("c", c_rank)]
     perm = [f"const int p_dim{i}" for i in range(pdims)]
     return f"void {func_name}({', '.join(ptrs + dims + perm + ['hipStream_t stream'])})"
+
+
+def uses_workspace(func_attrs: Dict[str, Any]) -> bool:
+    """The op's profiled instances asked for scratch memory (the profiler's WS field, kept as the op's
+    `workspace` attribute)."""
+    return int(func_attrs.get("workspace", 0) or 0) > 0
 
 
 def gemm_gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_dict) -> str:
@@ -228,15 +239,24 @@ def gemm_gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_i
     for key, item in func_attrs["exec_path"].items():
         if not item.algo:
             raise RuntimeError(f"{func_name}: workload {key} has no kernel instance; run profiling first")
+        if uses_workspace(func_attrs):
+            # a dynamic dim can ask for more scratch memory than the profiled sizes did: the library's own choice
+            # among the instances that fit takes over then
+            call = (f"aitamd_gemm_rcr_ws({epi}, {dtype}, "
+                    f"aitamd_gemm_workspace_bytes({epi}, {dtype}, algo, 1, M, N, K) <= workspace_bytes ? algo : -1, "
+                    f"a, b, {bias_arg}, {d0_arg}, {d1_arg}, c, M, N, K, "
+                    f"lda, ldb, ldc, ldd, workspace, workspace_bytes, stream)")
+        else:
+            call = (f"aitamd_gemm_rcr({epi}, {dtype}, algo, a, b, {bias_arg}, {d0_arg}, {d1_arg}, c, M, N, K, "
+                    f"lda, ldb, ldc, ldd, stream)")
         program = (
             f'static const int algo = resolve_instance({epi}, {dtype}, "{item.algo}");\n'
-            f"    check_rc(aitamd_gemm_rcr({epi}, {dtype}, algo, a, b, {bias_arg}, {d0_arg}, {d1_arg}, c, M, N, K, "
-            f'lda, ldb, ldc, ldd, stream), "{func_name}");'
+            f'    check_rc({call}, "{func_name}");'
         )
         launches.append(exec_cond_template.format(indent="  ", cond=item.exec_cond, program=program))
 
     return f"""{HEADER}
-{gemm_signature(func_name, op, a_rank, b_rank, c_rank)} {{
+{gemm_signature(func_name, op, a_rank, b_rank, c_rank, with_workspace=uses_workspace(func_attrs))} {{
 {shape_code}
   const {elem}* a = static_cast<const {elem}*>(in_ptr) + {off_a};
   const {elem}* b = static_cast<const {elem}*>(weight_ptr) + {off_b};
@@ -258,13 +278,17 @@ def gemm_func_decl(func_attrs: Dict[str, Any]) -> str:
     a_rank = len(func_attrs["input_accessors"][0].original_shapes)
     b_rank = len(func_attrs["input_accessors"][1].original_shapes)
     c_rank = len(func_attrs["output_accessors"][0].original_shapes)
-    return gemm_signature(func_attrs["name"], func_attrs["op"], a_rank, b_rank, c_rank) + ";"
+    return gemm_signature(func_attrs["name"], func_attrs["op"], a_rank, b_rank, c_rank,
+                          with_workspace=uses_workspace(func_attrs)) + ";"
 
 
 def gemm_func_call(func_attrs: Dict[str, Any], indent: str = "  ") -> str:
     """The call placed in the model's op list: tensor members, then the address of every dim member."""
     inputs, output = func_attrs["inputs"], func_attrs["outputs"][0]
     ptrs = [t._attrs["name"] for t in inputs[:2]] + [output._attrs["name"]] + [t._attrs["name"] for t in inputs[2:]]
+    if uses_workspace(func_attrs):
+        # every op gets the whole shared workspace: ops of one model run one after the other on its stream
+        ptrs += ["workspace_", "workspace_size_"]
     dims = []
     for acc in (func_attrs["input_accessors"][0], func_attrs["input_accessors"][1],
                 func_attrs["output_accessors"][0]):

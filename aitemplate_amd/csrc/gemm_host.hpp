@@ -18,9 +18,11 @@ struct GemmAlgo {
   int kvec;
   int lds_bytes;
   int wgs_per_cu;  // workgroups of this instance one CU holds at once
-  int direct_lds;  // 0: register-staged loads, 1: direct-to-LDS ring, 2: persistent direct-to-LDS ring
+  int direct_lds;  // 0: register-staged loads, 1: direct-to-LDS ring, 2: persistent direct-to-LDS ring, 4: 1 + split-K
   int layouts;     // bit L set: a kernel for operand layout L exists (0 rcr, 1 rrr, 2 ccr, 3 crr)
   hipError_t (*launch)(const GemmParams& p, hipStream_t stream);
+  // bytes of scratch memory (GemmParams::ws) a launch on this problem needs; null for instances that need none
+  int64_t (*workspace_bytes)(const GemmParams& p);
 };
 
 struct GemmAlgoTable {

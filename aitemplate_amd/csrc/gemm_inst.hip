@@ -44,10 +44,11 @@ template <class Tile, bool PERM, int LAYOUT>
 struct KernelOf {
   static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi, PERM, LAYOUT>;
 };
-template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, bool PERM, int LAYOUT>
-struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, PERM, LAYOUT> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, int SPLITK, bool PERM,
+          int LAYOUT>
+struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, SPLITK>, PERM, LAYOUT> {
   static constexpr auto value =
-      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>, Epi, PERM, LAYOUT>;
+      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, SPLITK>, Epi, PERM, LAYOUT>;
 };
 
 template <int BM, int BN, int BK, int WM, int WN, int NS, bool PERM, int LAYOUT>
@@ -66,9 +67,18 @@ struct LayoutMask<GemmTile<BM, BN, BK, WM, WN, 1>> {
   static constexpr int value = kLayoutBits;
 };
 template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
-struct LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>> {
+struct LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, 0>> {
   static constexpr int value =
       GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kTransposable ? kLayoutBits : 1;
+};
+// split-K form: rcr only
+template <class Tile>
+struct IsSplitK {
+  static constexpr bool value = false;
+};
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
+struct IsSplitK<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, 1>> {
+  static constexpr bool value = true;
 };
 template <class Tile>
 struct IsPersistent {
@@ -88,6 +98,31 @@ inline int device_cus(int dev) {
     cus[dev % kMaxDevices] = v;
   }
   return v;
+}
+
+// Workgroups per tile of a split-K launch: as many as bring the grid up to about one workgroup per CU, each with
+// at least two K-slabs, at most 16; 1 (no splitting, nothing written to the scratch memory) for grids that fill
+// the device anyway.
+template <class Tile>
+int split_k_factor(const GemmParams& p, int cus) {
+  const int64_t tiles = (int64_t)((p.M + Tile::BM - 1) / Tile::BM) * ((p.N + Tile::BN - 1) / Tile::BN) * p.batch;
+  const int64_t k_tiles = (p.K + Tile::BK - 1) / Tile::BK;
+  if (tiles <= 0) return 1;
+  int64_t s = cus / tiles;
+  if (s > k_tiles / 2) s = k_tiles / 2;
+  if (s > 16) s = 16;
+  return (int)(s < 1 ? 1 : s);
+}
+template <class Tile>
+int64_t workspace_of(const GemmParams& p) {
+  if constexpr (IsSplitK<Tile>::value) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const int64_t tiles = (int64_t)((p.M + Tile::BM - 1) / Tile::BM) * ((p.N + Tile::BN - 1) / Tile::BN) * p.batch;
+    const int s = split_k_factor<Tile>(p, device_cus(dev));
+    return s > 1 ? Tile::ws_bytes(tiles, s) : 0;
+  }
+  return 0;
 }
 
 template <class Tile, bool PERM, int LAYOUT = 0>
@@ -126,6 +161,14 @@ hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
   if constexpr (IsPersistent<Tile>::value) {
     const int cus = device_cus(dev);
     grid = dim3((unsigned)(total < cus ? total : cus), 1, 1);
+  }
+  if constexpr (IsSplitK<Tile>::value) {
+    // tiles are shared along K only with enough scratch memory to hold the partial tiles; without it the
+    // instance runs as its plain counterpart (one workgroup per tile, nothing written to the scratch memory)
+    p.split_k = split_k_factor<Tile>(p, device_cus(dev));
+    if (p.ws == nullptr || p.ws_bytes < Tile::ws_bytes(total, p.split_k) || total * p.split_k > 0x7fffffffll)
+      p.split_k = 1;
+    grid = dim3((unsigned)(total * p.split_k), 1, 1);
   }
   hipLaunchKernelGGL(kernel, grid, dim3(Tile::NT), Tile::kLdsBytes, stream, p);
   return hipGetLastError();
@@ -181,7 +224,7 @@ const GemmAlgo kAlgos[] = {
    BM, BN, BK, GemmTile<BM, BN, BK, WM, WN, KV>::NT, KV, GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes, \
    staged_wgs_per_cu(BM, BN, GemmTile<BM, BN, BK, WM, WN, KV>::NT,                                  \
                      GemmTile<BM, BN, BK, WM, WN, KV>::kLdsBytes),                                  \
-   0, LayoutMask<GemmTile<BM, BN, BK, WM, WN, KV>>::value, &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>},
+   0, LayoutMask<GemmTile<BM, BN, BK, WM, WN, KV>>::value, &launch_tile<GemmTile<BM, BN, BK, WM, WN, KV>>, nullptr},
 #define AITAMD_GEMM_TILE_DMA(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX)                                 \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
    "_c" #AUX,                                                                                              \
@@ -190,15 +233,25 @@ const GemmAlgo kAlgos[] = {
    dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::NT, OCC,                        \
                   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kLdsBytes),                      \
    1, LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>::value,                            \
-   &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>},
+   &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>, nullptr},
 #define AITAMD_GEMM_TILE_PERSIST(BM, BN, BK, WM, WN, NS)                                                  \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_persist" #NS,                      \
    BM, BN, BK, GemmTilePersist<BM, BN, BK, WM, WN, NS>::NT, 8, GemmTilePersist<BM, BN, BK, WM, WN, NS>::kLdsBytes, \
-   1, 2, 1, &launch_tile<GemmTilePersist<BM, BN, BK, WM, WN, NS>>},
+   1, 2, 1, &launch_tile<GemmTilePersist<BM, BN, BK, WM, WN, NS>>, nullptr},
+#define AITAMD_GEMM_TILE_DMA_SPLITK(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT)                                   \
+  {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
+   "_splitk",                                                                                             \
+   BM, BN, BK, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>::NT, 8,                             \
+   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>::kLdsBytes,                                     \
+   dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>::NT, OCC,                        \
+                  GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>::kLdsBytes),                      \
+   4, 1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>>,                             \
+   &workspace_of<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>>},
 #include "gemm_tiles.inc"
 #undef AITAMD_GEMM_TILE
 #undef AITAMD_GEMM_TILE_DMA
 #undef AITAMD_GEMM_TILE_PERSIST
+#undef AITAMD_GEMM_TILE_DMA_SPLITK
 };
 
 }  // namespace

@@ -53,6 +53,11 @@ struct GemmParams {
   // operand layout: 0 rcr (A [M, K], B [N, K]), 1 rrr (B [K, N]), 2 ccr (A [K, M]), 3 crr (both); lda / ldb
   // are the row pitches of the matrices as stored
   int32_t layout;
+  // Scratch memory of the split-K instances (null for every other instance): arrival counters, then slots for
+  // fp32 partial tiles; see gemm_kernel_dma.hpp.  The counters are zero before a launch and zero after it.
+  void* ws;
+  int64_t ws_bytes;
+  int32_t split_k;  // number of workgroups that share a tile along K (set by the launcher of a split-K instance)
 };
 
 AITAMD_DEVICE int64_t out_batch_offset(const GemmParams& p, int batch) {

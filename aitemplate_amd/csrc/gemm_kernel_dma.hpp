@@ -20,8 +20,22 @@
 
 namespace aitamd {
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int OCC_, int PIPE_ = 0, int MT_ = 32, int AUX_ = 0>
+// SPLITK_ = 1: GemmParams::split_k workgroups share each tile, each multiplying a contiguous part of the K-slabs;
+// every one of them leaves its fp32 partial tile in the scratch memory (GemmParams::ws) and counts itself on the
+// tile's counter, and the one that finds all the others counted sums the partial tiles in slab order (its own
+// included, so the result does not depend on who came last) and runs the epilogue.  Nobody waits for anybody.
+// For grids that leave most CUs idle and tiles small enough that a partial tile is a few KiB.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int OCC_, int PIPE_ = 0, int MT_ = 32, int AUX_ = 0,
+          int SPLITK_ = 0>
 struct GemmTileDma {
+  static constexpr int SPLITK = SPLITK_;
+  static constexpr int64_t kSlotBytes = (int64_t)BM_ * BN_ * 4;
+  static constexpr int64_t kCounterAlign = 4096;
+  // scratch bytes for `tiles` (batch x tile) pairs shared by `splits` workgroups each: one counter per pair,
+  // padded to 4 KiB, then one slot per workgroup
+  static constexpr int64_t ws_bytes(int64_t tiles, int splits) {
+    return SPLITK ? (tiles * 4 + kCounterAlign - 1) / kCounterAlign * kCounterAlign + tiles * splits * kSlotBytes : 0;
+  }
   // cache-policy bits of the slab loads: 1 = sc0, 2 = nt, 16 = sc1
   static constexpr int AUX = AUX_;
   // PIPE 0: barrier at the top of every K-slab.  PIPE 1: barrier inside the last
@@ -170,8 +184,12 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
   const int fr = lane % MT;  // row of the MFMA operand / column of the transposed result
   const int fq = lane / MT;  // which 8-wide k chunk of the MFMA step this lane feeds
 
+  // split-K: the workgroups of one split form one full grid of tiles (split s = workgroups [s * tiles, (s + 1) * tiles))
+  const int grid_tiles = p.tiles_m * p.tiles_n * p.batch;
+  const int split = Tile::SPLITK ? (int)blockIdx.x / grid_tiles : 0;
+  const int tile_wg = Tile::SPLITK ? (int)blockIdx.x - split * grid_tiles : (int)blockIdx.x;
   int batch, tm, tn;
-  map_tile<8>(blockIdx.x, p.tiles_m, p.tiles_n, p.batch, batch, tm, tn);
+  map_tile<8>(tile_wg, p.tiles_m, p.tiles_n, p.batch, batch, tm, tn);
   const int m0 = tm * BM;
   const int n0 = tn * BN;
   const int rows_a = (p.M - m0) < BM ? (p.M - m0) : BM;
@@ -236,7 +254,11 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
           (fq * 8 + (t_r >> 2)) * BN;
   }
 
-  const int k_tiles = (p.K + BK - 1) / BK;
+  const int k_tiles_all = (p.K + BK - 1) / BK;
+  // this workgroup's K-slabs [k_lo, k_lo + k_tiles)
+  const int splits = Tile::SPLITK ? p.split_k : 1;
+  const int k_lo = Tile::SPLITK ? (int)((int64_t)split * k_tiles_all / splits) : 0;
+  const int k_tiles = Tile::SPLITK ? (int)((int64_t)(split + 1) * k_tiles_all / splits) - k_lo : k_tiles_all;
 
   {
     // a transposed operand starts at its first column of the tile and ends with the tile's columns of row K-1
@@ -251,7 +273,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     // the end of K are still issued (every chunk out of range -> zero fill) so
     // the number of loads in flight per step stays constant for s_waitcnt.
     auto issue_loads = [&](int kt, int stage, int i0, int i1) {
-      const int k0 = kt * BK;
+      const int k0 = (Tile::SPLITK && kt >= k_tiles) ? p.K : (k_lo + kt) * BK;  // (past the own range: nothing to fetch)
       T* sbase = smem + stage * Tile::STAGE_ELEMS;
 #pragma unroll
       for (int i = 0; i < L_IT; ++i) {
@@ -385,6 +407,75 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     // drain the zero-fill slabs still in flight before LDS is reused
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
+
+    if constexpr (Tile::SPLITK != 0) {
+      // ---------------- split-K: partial tile to the scratch memory; the last workgroup of the tile sums ----
+      // ws: int32 counter per (batch, tile) pair, padded to 4 KiB, then slot (pair * splits + split) of BM * BN
+      // floats.  A lane's 16-byte pieces lie as ((wave * PIECES + q) * 64 + lane) * 16 bytes: every wave-store and
+      // wave-load is one contiguous KiB.  The slots may be read on another XCD than they were written on, whose L2
+      // does not see this one's lines: they are written through to memory and read from there (sc1), and a store
+      // is complete when vmcnt says so - no cache write-back or invalidate.
+      if (splits > 1) {
+        constexpr int PIECES = MI * NI * (ACC_N / 4);
+        constexpr int kCoherent = 16;
+        const int pair = batch * (p.tiles_m * p.tiles_n) + tm * p.tiles_n + tn;
+        int* const counters = reinterpret_cast<int*>(p.ws);
+        const int64_t counter_bytes = ((int64_t)grid_tiles * 4 + Tile::kCounterAlign - 1) / Tile::kCounterAlign * Tile::kCounterAlign;
+        unsigned char* const slots = reinterpret_cast<unsigned char*>(p.ws) + counter_bytes;
+        auto slot_rsrc = [&](int s_idx) {
+          const uint64_t a = reinterpret_cast<uint64_t>(slots + ((int64_t)pair * splits + s_idx) * Tile::kSlotBytes);
+          const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+          return make_rsrc(reinterpret_cast<void*>(((uint64_t)hi << 32) | lo), (uint32_t)Tile::kSlotBytes);
+        };
+        const uint32_t lane_off = (uint32_t)((wave * PIECES * 64 + lane) * 16);
+        {
+          const __amdgpu_buffer_rsrc_t rs = slot_rsrc(split);
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+              for (int q = 0; q < ACC_N / 4; ++q) {
+                f32x4 v4;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v4[j] = acc[mi][ni][q * 4 + j];
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v4), rs, lane_off,
+                                                       ((mi * NI + ni) * (ACC_N / 4) + q) * 1024, kCoherent);
+              }
+        }
+        wait_vmcnt<0>();  // this lane's part of the partial tile is in memory
+        __syncthreads();  // ... and so is every other lane's
+        int* const word = reinterpret_cast<int*>(smem_raw);
+        if (tid == 0) *word = __hip_atomic_fetch_add(&counters[pair], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __syncthreads();
+        const bool last = *word == splits - 1;
+        __syncthreads();
+        if (!last) return;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int e = 0; e < ACC_N; ++e) acc[mi][ni][e] = 0.0f;
+        for (int s_idx = 0; s_idx < splits; ++s_idx) {
+          const __amdgpu_buffer_rsrc_t rs = slot_rsrc(s_idx);
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+              for (int q = 0; q < ACC_N / 4; ++q) {
+                const f32x4 v4 = __builtin_bit_cast(
+                    f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, ((mi * NI + ni) * (ACC_N / 4) + q) * 1024, kCoherent));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[mi][ni][q * 4 + j] += v4[j];
+              }
+        }
+        // the counter is zero again for the next launch (which starts after this kernel has ended)
+        if (tid == 0) __hip_atomic_store(&counters[pair], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __syncthreads();  // (the broadcast word shares LDS with the epilogue's strips)
+      }
+    }
 
     // ---------------- epilogue: acc -> LDS (fp32, per-wave strip) -> 16-byte stores --------
     T* Cb = reinterpret_cast<T*>(p.c) + out_batch_offset(p, batch);

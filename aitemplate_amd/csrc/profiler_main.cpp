@@ -212,6 +212,10 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
   HIP_OK(hipEventCreate(&e0));
   HIP_OK(hipEventCreate(&e1));
 
+  // scratch memory of the instance being timed (the split-K ones; plain gemm_rcr ops only): zeroed once, the
+  // launches leave its counters zero
+  void* scratch = nullptr;
+  size_t scratch_bytes = 0;
   auto launch = [&](int algo, const OperandSet& o) -> int {
     if (perm.layout && !batched && perm.operands == AITAMD_LAYOUT_RCR)
       return aitamd_gemm_rcr_permute(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.c.p, M, N, K, K, K, perm.layout,
@@ -233,8 +237,8 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
       return aitamd_bmm_rcr_permute(dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, K, K, M * K, N * K, perm.g[0], stream);
     if (batched)
       return aitamd_bmm_rcr(dtype, algo, o.a.p, o.b.p, o.c.p, B, M, N, K, K, K, N, M * K, N * K, M * N, stream);
-    return aitamd_gemm_rcr(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.d0.p, o.d1.p, o.c.p, M, N, K, K, K, N, N,
-                           stream);
+    return aitamd_gemm_rcr_ws(epi, dtype, algo, o.a.p, o.b.p, o.bias.p, o.d0.p, o.d1.p, o.c.p, M, N, K, K, K, N, N,
+                              scratch, (int64_t)scratch_bytes, stream);
   };
 
   int printed = 0;
@@ -250,6 +254,18 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
     } else if (!aitamd_gemm_algo_supported(epi, dtype, algo, M, N, K, K, K, 16)) {
       continue;
     }
+    const bool plain = !batched && !perm.layout && perm.operands == AITAMD_LAYOUT_RCR;
+    const int64_t ws = plain ? aitamd_gemm_workspace_bytes(epi, dtype, algo, 1, M, N, K) : 0;
+    if (!plain && strstr(name, "_splitk")) continue;  // (the other entry points take no scratch memory)
+    if (scratch) HIP_OK(hipFree(scratch));
+    scratch = nullptr;
+    scratch_bytes = (size_t)ws;
+    if (ws > 0) {
+      HIP_OK(hipMalloc(&scratch, scratch_bytes));
+      HIP_OK(hipMemset(scratch, 0, scratch_bytes));
+    } else if (strstr(name, "_splitk")) {
+      continue;  // does not split on this problem: the same as the plain instance, which is timed anyway
+    }
     bool ok = true;
     for (int i = 0; i < warmup && ok; ++i) ok = launch(algo, pool[i % sets]) == 0;
     if (!ok) {
@@ -263,10 +279,11 @@ int profile_gemm_like(const std::string& op, int dtype, int64_t B, int64_t M, in
     HIP_OK(hipEventSynchronize(e1));
     float ms = 0.f;
     HIP_OK(hipEventElapsedTime(&ms, e0, e1));
-    printf("OP:%s,TIME:%.6f,WS:0\n", name, ms / (iters > 0 ? iters : 1));
+    printf("OP:%s,TIME:%.6f,WS:%lld\n", name, ms / (iters > 0 ? iters : 1), (long long)ws);
     fflush(stdout);
     ++printed;
   }
+  if (scratch) HIP_OK(hipFree(scratch));
   HIP_OK(hipStreamDestroy(stream));
   return printed > 0 ? 0 : 3;
 }

@@ -42,14 +42,28 @@ def _row_pitch(t: torch.Tensor, name: str) -> int:
     return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], t.stride(0))
 
 
+def gemm_workspace_bytes(op: str, algo: int, M: int, N: int, K: int, dtype=torch.float16, batch: int = 1) -> int:
+    """Bytes of scratch memory instance `algo` of `op` needs for this problem (0 for all but the split-K ones)."""
+    lib = _kernels.load()
+    return int(lib.aitamd_gemm_workspace_bytes(_kernels.EPILOGUE_OF_OP[op], _TORCH_DTYPE_ID[dtype], algo, batch, M, N, K))
+
+
+def new_workspace(nbytes: int, device="cuda") -> torch.Tensor:
+    """A scratch buffer for `gemm(..., workspace=)`: zeroed once (the kernels leave its counters zero again)."""
+    return torch.zeros(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
 def gemm(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None,
          d0: Optional[torch.Tensor] = None, d1: Optional[torch.Tensor] = None,
-         out: Optional[torch.Tensor] = None, algo: int = -1) -> torch.Tensor:
+         out: Optional[torch.Tensor] = None, algo: int = -1,
+         workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Run reference op `op` (e.g. "gemm_rcr_bias_gelu"): out = epilogue(a @ b.T, bias, d0, d1).
 
     `a` may have more than 2 dims; leading dims are flattened into M as the
     reference does (gemm_rcr.py:51-77).  `algo` = -1 uses the library heuristic,
-    otherwise the instance index (see `_kernels.gemm_algo_names`).
+    otherwise the instance index (see `_kernels.gemm_algo_names`).  `workspace`: a buffer from
+    `new_workspace` for the instances that split K between workgroups (the reference ops' `workspace`
+    attribute, gemm_common.py:201-215); without it those instances are not chosen.
     """
     lib = _kernels.load()
     epi = _kernels.EPILOGUE_OF_OP[op]
@@ -86,9 +100,12 @@ def gemm(op: str, a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor]
     ldd = _row_pitch(d0_2, "d0") if nres >= 1 else N
     if nres >= 2 and _row_pitch(d1_2, "d1") != ldd:
         raise ValueError("d0 and d1 must share a row pitch")
-    rc = lib.aitamd_gemm_rcr(epi, _TORCH_DTYPE_ID[dtype], algo, _p(a2), _p(b), _p(bias), _p(d0_2), _p(d1_2),
-                             _p(out2), M, N, K, _row_pitch(a2, "a"), _row_pitch(b, "b"), _row_pitch(out2, "out"),
-                             ldd, _stream_ptr())
+    if workspace is not None and (not workspace.is_cuda or not workspace.is_contiguous()
+                                  or workspace.dtype != torch.uint8):
+        raise ValueError("workspace must be a contiguous uint8 GPU tensor (see new_workspace)")
+    rc = lib.aitamd_gemm_rcr_ws(epi, _TORCH_DTYPE_ID[dtype], algo, _p(a2), _p(b), _p(bias), _p(d0_2), _p(d1_2),
+                                _p(out2), M, N, K, _row_pitch(a2, "a"), _row_pitch(b, "b"), _row_pitch(out2, "out"),
+                                ldd, _p(workspace), 0 if workspace is None else workspace.numel(), _stream_ptr())
     _kernels.check(rc, op)
     return out
 

@@ -32,7 +32,13 @@ ModelBase::ModelBase(size_t blob_size, size_t workspace_size, size_t num_inputs,
   AIT_DEVICE_CHECK(hipGetDevice(&device_idx_));
   AIT_DEVICE_CHECK(hipEventCreateWithFlags(&run_finished_, hipEventDisableTiming));
   if (blob_size > 0) blob_ = static_cast<uint8_t*>(allocator_.Allocate(blob_size));
-  if (workspace_size > 0) workspace_ = static_cast<uint8_t*>(allocator_.Allocate(workspace_size));
+  if (workspace_size > 0) {
+    // Scratch memory shared by the ops that need some (split-K GEMM instances).  Their arrival counters must be
+    // zero before the first launch and every launch leaves them zero, so the buffer is cleared once, here.
+    workspace_ = static_cast<uint8_t*>(allocator_.Allocate(workspace_size));
+    workspace_size_ = static_cast<int64_t>(workspace_size);
+    AIT_DEVICE_CHECK(hipMemset(workspace_, 0, workspace_size));
+  }
 }
 
 ModelBase::~ModelBase() {

@@ -118,6 +118,7 @@ class ModelBase {
   std::vector<OpEntry> ops_;
   uint8_t* blob_ = nullptr;
   uint8_t* workspace_ = nullptr;
+  int64_t workspace_size_ = 0;
   uint8_t* constants_ = nullptr;
   size_t num_inputs_;
   size_t num_outputs_;

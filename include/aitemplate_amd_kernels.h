@@ -111,6 +111,29 @@ AITAMD_API int aitamd_gemm_rcr(int epilogue, int dtype, int algo,
                                int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
                                void* stream);
 
+/* Scratch memory for instances that split tiles between workgroups along K (the "splitk" instances): bytes that
+ * instance `algo` needs for this problem on the current device, 0 for every other instance.  The reference's ops
+ * carry the same quantity as their `workspace` attribute, filled from the profiler's WS:<bytes> field
+ * (python/aitemplate/compiler/ops/gemm_universal/gemm_common.py:201-215, 566-569) and served from the model's one
+ * shared workspace (python/aitemplate/compiler/transform/memory_planning.py:155-194). */
+AITAMD_API int64_t aitamd_gemm_workspace_bytes(int epilogue, int dtype, int algo, int64_t batch,
+                                               int64_t M, int64_t N, int64_t K);
+
+/* aitamd_gemm_rcr with scratch memory: `workspace` is device memory, 16-byte aligned, of `workspace_bytes` bytes.
+ * Its first 4096 bytes must be zero before the first launch that uses the buffer; every launch leaves them zero
+ * again, so one memset after allocation serves any number of launches.  Launches that overlap in time (different
+ * streams) need buffers of their own.  algo = -1 may then choose a splitk instance; a splitk instance that gets no
+ * buffer, or one smaller than aitamd_gemm_workspace_bytes says, runs without sharing tiles (as the plain instance of
+ * the same tile, touching no scratch memory); instances that need no scratch memory ignore the buffer.
+ * Same role as the generated op functions' `workspace` argument in the reference
+ * (python/aitemplate/backend/rocm/gemm/common.py:491-521, func_call with the global workspace pointer). */
+AITAMD_API int aitamd_gemm_rcr_ws(int epilogue, int dtype, int algo,
+                                  const void* a, const void* b, const void* bias,
+                                  const void* d0, const void* d1, void* c,
+                                  int64_t M, int64_t N, int64_t K,
+                                  int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                                  void* workspace, int64_t workspace_bytes, void* stream);
+
 /* gemm_rcr[_bias...] whose [M, N] result is written through one of the reference's 5-D output permutations
  * into a contiguous buffer.  Epilogues AITAMD_EPI_NONE and AITAMD_EPI_BIAS only (the ones the permuting ops use);
  * g = (g1, g2, g3) is the op's `shape` attribute.

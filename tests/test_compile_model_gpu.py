@@ -69,6 +69,35 @@ def _run_gemm_case(op_name, Ms, N, K, dtype="float16", tol=1e-2):
     module.close()
 
 
+def test_split_k_instance_through_compile_model():
+    """A few tiles with a very long K: the profiler finds a split-K instance fastest, its WS:<bytes> becomes the
+    op's `workspace` attribute, the model allocates that once and hands it to the op function (the reference's
+    workspace path: gemm_common.py:201-215, 566-569; memory_planning.py:155-194).  A dynamic M between the profiled
+    sizes runs too."""
+    op_name, Ms, N, K = "gemm_rcr_bias", [64, 128], 256, 8192
+    m_dim = shape_utils.gen_int_var_min_max(Ms, name="m")
+    X = Tensor(shape=[m_dim, IntImm(K)], dtype="float16", name="input_0", is_input=True)
+    W = Tensor(shape=[IntImm(N), IntImm(K)], dtype="float16", name="input_1", is_input=True)
+    B = Tensor(shape=[IntImm(N)], dtype="float16", name="input_2", is_input=True)
+    op = ops.gemm_rcr_bias()
+    Y = _mark_output(op(X, W, B))
+    module = compile_model(Y, detect_target(), WORKDIR, f"split_k_{next(_counter)}", num_runtimes=2)
+    algos = [item.algo for item in op._attrs["exec_path"].values()]
+    print("chosen:", algos, "workspace:", op._attrs["workspace"], flush=True)
+    if os.environ.get("CI_FLAG") != "CIRCLECI":  # (without timing the heuristic has no scratch memory to offer)
+        assert any(a.endswith("_splitk") for a in algos), algos
+        assert op._attrs["workspace"] > 0
+    for M in (64, 100, 128):
+        x, w, b = _rand((M, K), 1), _rand((N, K), 2, K ** -0.5), _rand((N,), 3)
+        want = oracle.torch_gemm(op_name, x, w, b).half().float()
+        for rep in range(2):
+            y = torch.empty(M, N, dtype=torch.float16, device="cuda")
+            module.run_with_tensors({"input_0": x.cuda(), "input_1": w.cuda(), "input_2": b.cuda()}, [y],
+                                    graph_mode=rep == 1)
+            torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    module.close()
+
+
 def test_gemm_rcr_simple_static():          # test_gemm.py:83-84
     _run_gemm_case("gemm_rcr", [1024], 512, 256)
 
