@@ -87,6 +87,8 @@ EXPORTED_SYMBOLS = [
     "aitamd_attention_set_variant",
     "aitamd_gemm_workspace_bytes",
     "aitamd_gemm_rcr_ws",
+    "aitamd_gemm_rcr_noalloc",
+    "aitamd_gemm_noalloc_scratch_bytes",
 ]
 
 _lock = threading.Lock()
@@ -152,6 +154,10 @@ def load() -> ctypes.CDLL:
         lib.aitamd_gemm_workspace_bytes.argtypes = [i32, i32, i32, i64, i64, i64, i64]
         lib.aitamd_gemm_rcr_ws.restype = i32
         lib.aitamd_gemm_rcr_ws.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp, i64, vp]
+        lib.aitamd_gemm_rcr_noalloc.restype = i32
+        lib.aitamd_gemm_rcr_noalloc.argtypes = [i32, i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp]
+        lib.aitamd_gemm_noalloc_scratch_bytes.restype = i64
+        lib.aitamd_gemm_noalloc_scratch_bytes.argtypes = []
         lib.aitamd_attention_set_variant.restype = i32
         lib.aitamd_attention_set_variant.argtypes = [i32]
         _lib = lib

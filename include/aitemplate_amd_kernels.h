@@ -134,6 +134,20 @@ AITAMD_API int aitamd_gemm_rcr_ws(int epilogue, int dtype, int algo,
                                   int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
                                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* aitamd_gemm_rcr_ws for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc): the scratch memory is a 16 MiB array inside the library's device image, one per GPU, held
+ * from the first call on that GPU until the process ends; the call itself allocates and frees nothing.  It has no
+ * counterpart in the reference (whose ops draw their workspace from the model's allocation).  An instance named by
+ * `algo` that needs more than aitamd_gemm_noalloc_scratch_bytes() for this problem is refused with a message;
+ * algo = -1 chooses among the instances that fit.  All calls on one GPU share that GPU's array: calls that overlap
+ * in time on one GPU (different streams) race - serialise them, or use aitamd_gemm_rcr_ws with separate buffers. */
+AITAMD_API int aitamd_gemm_rcr_noalloc(int epilogue, int dtype, int algo,
+                                       const void* a, const void* b, const void* bias,
+                                       const void* d0, const void* d1, void* c,
+                                       int64_t M, int64_t N, int64_t K,
+                                       int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd, void* stream);
+AITAMD_API int64_t aitamd_gemm_noalloc_scratch_bytes(void);
+
 /* gemm_rcr[_bias...] whose [M, N] result is written through one of the reference's 5-D output permutations
  * into a contiguous buffer.  Epilogues AITAMD_EPI_NONE and AITAMD_EPI_BIAS only (the ones the permuting ops use);
  * g = (g1, g2, g3) is the op's `shape` attribute.
