@@ -153,7 +153,7 @@ def gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_info_d
             f'    check_rc({call}, "{func_name}");'
         )
         launches.append(exec_cond_template.format(indent="  ", cond=item.exec_cond, program=program))
-    return f"""{common.HEADER}
+    return f"""{common.header_with_table(epi, dtype)}
 {_signature(func_name, (ra, rb, rc), permute, add)} {{
 {shape_code}
   const uint16_t* a = static_cast<const uint16_t*>(in_ptr) + {off_a};

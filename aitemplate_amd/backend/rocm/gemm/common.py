@@ -188,6 +188,15 @@ namespace ait {
 FOOTER = "\n}  // namespace ait\n"
 
 
+def header_with_table(epilogue: int, dtype: int) -> str:
+    """HEADER plus a reference that makes the linker take the instance table of (epilogue, dtype) out of the
+    kernel archive: a model library carries the kernels of the tables its op functions name, nothing else."""
+    sym = f"aitamd_gemm_table_{epilogue}_{dtype}"
+    ref = (f'extern "C" void {sym}();\n'
+           f"namespace {{\n__attribute__((used)) void (*const keep_{sym})() = &{sym};\n}}  // namespace\n")
+    return HEADER.replace("\nnamespace ait {\n", "\n" + ref + "\nnamespace ait {\n")
+
+
 def gemm_signature(func_name: str, op_name: str, a_rank: int, b_rank: int, c_rank: int, pdims: int = 0,
                    with_workspace: bool = False) -> str:
     """Launcher prototype; `pdims` trailing `const int p_dim<i>` carry a permuting op's shape attribute
@@ -255,7 +264,7 @@ def gemm_gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_i
         )
         launches.append(exec_cond_template.format(indent="  ", cond=item.exec_cond, program=program))
 
-    return f"""{HEADER}
+    return f"""{header_with_table(epi, dtype)}
 {gemm_signature(func_name, op, a_rank, b_rank, c_rank, with_workspace=uses_workspace(func_attrs))} {{
 {shape_code}
   const {elem}* a = static_cast<const {elem}*>(in_ptr) + {off_a};

@@ -63,14 +63,21 @@ class ROCM(Target):
         return f"{self.cc()} {opts} -c -o {{target}} {{src}}"
 
     def link_options(self, shared: bool = True) -> str:
+        """A model library is self-contained: the runtime archive whole, and from the kernel archive the objects
+        its op functions refer to (each names the instance table it dispatches through).  Nothing points back
+        into this source tree; the only shared libraries it needs are the HIP runtime and the C++ runtime
+        (reference: backend/builder.py:398-527, where everything is linked into test.so)."""
         flags = ["-shared"] if shared else []
         flags += [
             f"-L{LIB_PATH}",
-            # the archive's C ABI objects are referenced by nobody inside the library: keep all of it
+            # the runtime archive's C ABI objects are referenced by nobody inside the library: keep all of it
             "-Wl,--whole-archive -laitemplate_amd_runtime -Wl,--no-whole-archive" if shared else "",
-            "-laitemplate_amd_kernels",
+            "-l:libaitemplate_amd_kernels_static.a",
+            # the kernel entry points stay private to the model library (a process may hold several model
+            # libraries and the shared kernel library at once)
+            "-Wl,--exclude-libs,libaitemplate_amd_kernels_static.a",
             f"-L{self._rocm_path}/lib", "-lamdhip64", "-lpthread",
-            f"-Wl,-rpath,{LIB_PATH}", f"-Wl,-rpath,{self._rocm_path}/lib",
+            f"-Wl,-rpath,{self._rocm_path}/lib",
         ]
         return " ".join(f for f in flags if f)
 

@@ -1,6 +1,7 @@
 // C ABI launcher of the fused attention kernel (bmm_softmax_bmm_permute).
 #include <atomic>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 
 #include "../../include/aitemplate_amd_kernels.h"
@@ -107,9 +108,40 @@ AttnLaunch pick(int ks, int ot) {
   return nullptr;
 }
 
+// x rounded to the nearest fp16 (dtype 0) or bf16 value, ties to even, as a float.  Done on the bits: host-side
+// conversions through _Float16 / __bf16 would call compiler-runtime routines that a model library linked by the
+// host C++ compiler does not have.
 float round_to_elem(float x, int dtype) {
-  if (dtype == 0) return (float)(_Float16)x;
-  return (float)(__bf16)x;
+  uint32_t u;
+  memcpy(&u, &x, 4);
+  const uint32_t sign = u & 0x80000000u, mag = u & 0x7fffffffu;
+  if (mag >= 0x7f800000u) return x;  // infinities and NaNs stay what they are
+  uint32_t r;
+  if (dtype != 0) {
+    r = mag + 0x7fffu + ((mag >> 16) & 1u);  // keep 8 bits of mantissa
+    r &= 0xffff0000u;
+  } else {
+    const int e = (int)(mag >> 23) - 127;
+    if (e > 15) {
+      r = 0x7f800000u;  // beyond the largest half
+    } else if (e >= -14) {
+      r = mag + 0xfffu + ((mag >> 13) & 1u);  // normal half: keep 10 bits of mantissa
+      r &= 0xffffe000u;
+      if (r >= 0x47800000u) r = 0x7f800000u;  // rounded up past 65504
+    } else {
+      // subnormal half: a multiple of 2^-24
+      float f;
+      memcpy(&f, &mag, 4);
+      const float q = f * 16777216.0f;          // exact scaling
+      const float n = __builtin_rintf(q);       // ties to even in the default rounding mode
+      f = n * (1.0f / 16777216.0f);
+      memcpy(&r, &f, 4);
+    }
+  }
+  r |= sign;
+  float out;
+  memcpy(&out, &r, 4);
+  return out;
 }
 
 }  // namespace

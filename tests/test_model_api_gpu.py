@@ -294,6 +294,34 @@ def test_bound_constant_double_buffer_takes_effect_at_the_swap():
     mod.close()
 
 
+def test_model_library_is_self_contained(tmp_path):
+    """test.so copied away from its build directory - alone - loads and runs: it carries the runtime and the kernels
+    of the instance tables its ops use, and needs no other file of this package (the reference links everything into
+    test.so as well, backend/builder.py:398-527)."""
+    import shutil
+    import subprocess
+
+    mod = compile_model(_graph(), detect_target(), WORKDIR, "model_api_portable")
+    mod.close()
+    built = os.path.join(WORKDIR, "model_api_portable", "test.so")
+    lone = tmp_path / "elsewhere" / "model.so"
+    lone.parent.mkdir()
+    shutil.copy2(built, lone)
+    needed = subprocess.run(["ldd", str(lone)], capture_output=True, text=True).stdout
+    assert "aitemplate_amd" not in needed, needed
+    assert "not found" not in needed, needed
+    assert "libamdhip64" in needed
+    dynamic = subprocess.run(["readelf", "-d", str(lone)], capture_output=True, text=True).stdout
+    assert "aitemplate_amd" not in dynamic, dynamic  # no run path into the source tree either
+    # one (epilogue, dtype) table of kernels, not the whole 30 MB library
+    assert os.path.getsize(lone) < 8 << 20
+    x, w, b, want = _data(16)
+    y = torch.empty(16, N, dtype=torch.float16, device="cuda")
+    with Model(str(lone)) as portable:
+        portable.run_with_tensors([x.cuda(), w.cuda(), b.cuda()], [y])
+    torch.testing.assert_close(y.cpu().float(), want, atol=1e-2, rtol=1e-2)
+
+
 def test_ait_recompile_0_loads_existing_library(module, monkeypatch):
     monkeypatch.setenv("AIT_RECOMPILE", "0")
     mod = compile_model(_graph(), detect_target(), WORKDIR, "model_api_simple")
