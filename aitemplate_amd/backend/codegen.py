@@ -94,6 +94,16 @@ class ModelSource:
                 seen_dims.add(n)
                 init = d.value() if isinstance(d, IntImm) else d.upper_bound()
                 lines.append(f"  int64_t {n} {{{init}}};")
+        # dims of views that a split / concatenate fusion left only in an op's accessor
+        for op in get_sorted_ops(self.graph):
+            for acc in (op._attrs.get("input_accessors") or []) + (op._attrs.get("output_accessors") or []):
+                for d in acc.original_shapes:
+                    n = d._attrs["name"]
+                    if n in seen_dims:
+                        continue
+                    seen_dims.add(n)
+                    init = d.value() if isinstance(d, IntImm) else d.upper_bound()
+                    lines.append(f"  int64_t {n} {{{init}}};")
         return "\n".join(lines)
 
     def param_table(self) -> str:

@@ -236,13 +236,34 @@ def gemm_gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_i
     bias_arg = "bias_ptr" if "bias_ptr" in extras else "nullptr"
     d0_arg = "d0_ptr" if "d0_ptr" in extras else "nullptr"
     d1_arg = "d1_ptr" if "d1_ptr" in extras else "nullptr"
-    # residual tensors may be strided views as well
+    # residual tensors may be strided views as well: each has its own offset, both share one row pitch
     ldd = "N"
-    n_in = len(func_attrs["inputs"])
-    if n_in > 3:
-        _, p = accessor_offset_and_pitch(func_attrs["input_accessors"][3], "d0")
-        if p is not None:
-            ldd = str(p)
+    res_offsets = {}
+    pitches = set()
+    for name in extras:
+        if name == "bias_ptr":
+            continue
+        off_d, p = accessor_offset_and_pitch(func_attrs["input_accessors"][2 + extras.index(name)], name)
+        res_offsets[name] = off_d
+        pitches.add(p)
+    if len(pitches) > 1:
+        raise NotImplementedError(f"{op}: the two residuals must have the same row pitch, got {sorted(map(str, pitches))}")
+    if pitches and next(iter(pitches)) is not None:
+        ldd = str(next(iter(pitches)))
+    if "bias_ptr" in extras:
+        b_off, b_pitch = accessor_offset_and_pitch(func_attrs["input_accessors"][2], "bias")
+        if b_off or b_pitch is not None:
+            raise NotImplementedError(f"{op}: the bias cannot be a view of a wider tensor")
+    if d0_arg != "nullptr":
+        d0_arg = "d0"
+    if d1_arg != "nullptr":
+        d1_arg = "d1"
+    residual_ptrs = "".join(
+        f"  const {elem}* {n[:-4]} = static_cast<const {elem}*>({n}) + {res_offsets[n]};\n" for n in res_offsets)
+    # The instance was profiled on contiguous operands.  A view whose offset or pitch is not a whole number of
+    # 16-byte pieces can rule that instance out; the library then picks among the instances that fit.
+    misaligned = any(v % 8 for v in (off_a, off_b, lda or 0, ldb or 0))
+    algo_expr = "-1" if misaligned else "algo"
 
     launches = []
     for key, item in func_attrs["exec_path"].items():
@@ -252,11 +273,11 @@ def gemm_gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_i
             # a dynamic dim can ask for more scratch memory than the profiled sizes did: the library's own choice
             # among the instances that fit takes over then
             call = (f"aitamd_gemm_rcr_ws({epi}, {dtype}, "
-                    f"aitamd_gemm_workspace_bytes({epi}, {dtype}, algo, 1, M, N, K) <= workspace_bytes ? algo : -1, "
+                    f"aitamd_gemm_workspace_bytes({epi}, {dtype}, algo, 1, M, N, K) <= workspace_bytes ? {algo_expr} : -1, "
                     f"a, b, {bias_arg}, {d0_arg}, {d1_arg}, c, M, N, K, "
                     f"lda, ldb, ldc, ldd, workspace, workspace_bytes, stream)")
         else:
-            call = (f"aitamd_gemm_rcr({epi}, {dtype}, algo, a, b, {bias_arg}, {d0_arg}, {d1_arg}, c, M, N, K, "
+            call = (f"aitamd_gemm_rcr({epi}, {dtype}, {algo_expr}, a, b, {bias_arg}, {d0_arg}, {d1_arg}, c, M, N, K, "
                     f"lda, ldb, ldc, ldd, stream)")
         program = (
             f'static const int algo = resolve_instance({epi}, {dtype}, "{item.algo}");\n'
@@ -270,7 +291,7 @@ def gemm_gen_function(func_attrs: Dict[str, Any], exec_cond_template: str, dim_i
   const {elem}* a = static_cast<const {elem}*>(in_ptr) + {off_a};
   const {elem}* b = static_cast<const {elem}*>(weight_ptr) + {off_b};
   {elem}* c = static_cast<{elem}*>(out_ptr) + {off_c};
-  const int64_t lda = {lda if lda is not None else "K"};
+{residual_ptrs}  const int64_t lda = {lda if lda is not None else "K"};
   const int64_t ldb = {ldb if ldb is not None else "K"};
   const int64_t ldc = {ldc if ldc is not None else "N"};
   const int64_t ldd = {ldd};

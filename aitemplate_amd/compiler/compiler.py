@@ -76,6 +76,8 @@ def compile_model(
             if do_optimize_graph:
                 graph = transform.fuse_mm_elementwise(graph, output_tensors)
             transform.check_no_elementwise_left(graph)
+            # last-dim split / concatenate become offsets and row pitches of the GEMM ops around them
+            graph = transform.fuse_strided_views(graph, output_tensors)
             transform.name_graph(graph)
             transform.mark_param_tensor(graph, output_tensors)
             transform.profile(graph, profile_dir, profile_devs, dynamic_profiling_strategy, profile_timeout)

@@ -1,9 +1,14 @@
-"""View ops: reshape (and flatten via reshape) and split along the outermost dim — outputs alias their
-input's memory.
+"""View ops: reshape (and flatten via reshape), split and concatenate — ops that move no data on this
+backend.
 
 Counterpart of the reshape in python/aitemplate/compiler/ops/common/view_ops.py, reduced
-to static target shapes with at most one -1 (what the GEMM-family graphs use), and of
-python/aitemplate/compiler/ops/tensor/split.py:31-170 for the case that needs no copy."""
+to static target shapes with at most one -1 (what the GEMM-family graphs use), of
+python/aitemplate/compiler/ops/tensor/split.py:31-170 and of
+python/aitemplate/compiler/ops/tensor/concatenate.py:31-170 for the cases that need no copy:
+an outer-dim split is a byte offset into its input; a last-dim split or concatenate only
+exists until the strided-view pass has turned it into offsets and row pitches of the GEMM
+ops on either side (the reference's transform_strided_ops.py does the same, and falls back
+to a copy kernel where this backend raises)."""
 from typing import List, Sequence, Union
 
 from ...base import IntImm, IntVar, Operator, Tensor
@@ -92,11 +97,14 @@ class flatten(reshape):
 class split(_view):
     """torch.split(x, split_size_or_sections, dim) -> tuple of tensors.
 
-    Only splits that leave every piece contiguous are supported (dim 0, or a dim preceded by dims of
-    size 1) with static shapes: each piece is then a view at a byte offset into x and no kernel runs.
-    This is the split nn.MultiheadAttention applies to the packed [3, batch, heads, seq, head_dim]
-    projection.  The reference materialises every split with a copy kernel unless a later pass removes
-    it (split.py:172-214)."""
+    Two kinds of split run no kernel here.  A split that leaves every piece contiguous (dim 0, or a
+    dim preceded by dims of size 1, static shapes) makes each piece a view at a byte offset into x:
+    the split nn.MultiheadAttention applies to the packed [3, batch, heads, seq, head_dim]
+    projection.  A split along the last dim makes pieces that are strided views (`strided_view_of`
+    = (x, dim, first element)); every consumer has to be an op that can read an operand through an
+    offset and a row pitch, and the strided-view pass of compile_model rewires them to x.  The
+    reference materialises every split with a copy kernel unless a later pass removes it
+    (split.py:172-214)."""
 
     def __init__(self):
         super().__init__()
@@ -112,11 +120,12 @@ class split(_view):
         if not -rank <= dim < rank:
             raise RuntimeError(f"split dim ({dim}) expected to be less than rank ({rank})")
         dim %= rank
-        if not all(isinstance(d, IntImm) for d in shape):
-            raise NotImplementedError("split needs static shapes on this backend")
-        if any(d.value() != 1 for d in shape[:dim]):
-            raise NotImplementedError("split along an inner dim would need a copy kernel; only dim 0 "
-                                      "(or a dim behind dims of size 1) is supported")
+        if not all(isinstance(d, IntImm) for d in shape[dim:]):
+            raise NotImplementedError("split needs static shapes from the split dim on")
+        contiguous = all(isinstance(d, IntImm) and d.value() == 1 for d in shape[:dim])
+        if not contiguous and dim != rank - 1:
+            raise NotImplementedError("split along a middle dim would need a copy kernel; only dim 0 (or a dim "
+                                      "behind dims of size 1) and the last dim are supported")
         size = shape[dim].value()
         if isinstance(split_size_or_sections, (list, tuple)):
             sizes = [int(v.value()) if isinstance(v, IntImm) else int(v) for v in split_size_or_sections]
@@ -146,11 +155,64 @@ class split(_view):
         for n in sizes:
             out_shape = list(shape[:dim]) + [IntImm(n)] + list(shape[dim + 1:])
             t = Tensor(out_shape, src_ops={self}, is_view_of=x, dtype=x.dtype())
-            t._attrs["view_offset_bytes"] = start * inner
+            if contiguous:
+                t._attrs["view_offset_bytes"] = start * inner
+            else:
+                t._attrs["strided_view_of"] = (x, dim, start)
             outputs.append(t)
             start += n
         self._attrs["outputs"] = outputs
         return tuple(outputs)
+
+    def _get_op_attributes(self):
+        return {}
+
+
+class concatenate(_view):
+    """torch.cat(tensors, dim) along the last dim, for inputs that GEMM-family ops write.
+
+    The op is a placeholder: the strided-view pass of compile_model makes every producer write its
+    columns of the output directly (offset + row pitch of its C accessor) and drops the op.  An
+    input that no such op produces (a graph input, a constant, a tensor with other consumers) would
+    need the reference's copy kernel (backend/rocm/tensor/concatenate.py) and raises there."""
+
+    def __init__(self):
+        super().__init__()
+        self._attrs["op"] = "concatenate"
+        self._attrs["is_view_op"] = True
+        self._attrs["has_profiler"] = False
+
+    def __call__(self, inputs: Sequence[Tensor], dim: int = -1) -> Tensor:
+        inputs = list(inputs)
+        if len(inputs) < 1:
+            raise RuntimeError("concatenate expects at least one tensor")
+        rank = inputs[0]._rank()
+        if not -rank <= dim < rank:
+            raise RuntimeError(f"concatenate dim ({dim}) expected to be less than rank ({rank})")
+        dim %= rank
+        if dim != rank - 1:
+            raise NotImplementedError("concatenate along a dim other than the last would need a copy kernel")
+        first = inputs[0]._attrs["shape"]
+        total = 0
+        for t in inputs:
+            shape = t._attrs["shape"]
+            if len(shape) != rank:
+                raise RuntimeError("concatenate expects tensors of the same rank")
+            if t.dtype() != inputs[0].dtype():
+                raise RuntimeError("concatenate expects tensors of the same dtype")
+            for i, (d0, d1) in enumerate(zip(first, shape)):
+                if i != dim and d0 != d1:
+                    raise RuntimeError(f"concatenate: dim {i} differs between inputs ({d0} vs {d1})")
+            if not isinstance(shape[dim], IntImm):
+                raise NotImplementedError("concatenate needs a static size along the concatenated dim")
+            total += shape[dim].value()
+        self._attrs["inputs"] = inputs
+        self._attrs["concat_dim"] = dim
+        self._set_depth()
+        out_shape = list(first[:dim]) + [IntImm(total)] + list(first[dim + 1:])
+        output = Tensor(out_shape, src_ops={self}, dtype=inputs[0].dtype())
+        self._attrs["outputs"] = [output]
+        return output
 
     def _get_op_attributes(self):
         return {}

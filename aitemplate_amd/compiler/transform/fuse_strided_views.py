@@ -1,0 +1,140 @@
+"""Turn last-dim split / concatenate ops into offsets and row pitches of the GEMM ops around them.
+
+Counterpart of python/aitemplate/compiler/transform/transform_strided_ops.py:33-64 with its two
+rewrites that matter for the GEMM family:
+
+* split + strided op (transform_strided_ops.py `_fuse_split_and_strided_op`): an op that reads a
+  piece of a last-dim split reads the split's input instead, through
+  `input_accessors[i].update_base_tensor(x, dim, first element)`; when every piece has been
+  rewired the split leaves the graph.
+* strided op + concatenate (transform_strided_ops.py `_fuse_strided_op_and_cat`): an op whose
+  output feeds a last-dim concatenate writes its columns of the concatenated tensor directly,
+  through `output_accessors[0].update_base_tensor(cat_output, dim, first element)`; the
+  concatenate leaves the graph and its output has one producer per input.
+
+The reference keeps a split or concatenate it cannot fuse and runs a copy kernel for it.  This
+backend has GEMM-family kernels only, so a piece whose consumer (or producer) cannot take a view
+raises NotImplementedError, naming the tensor and the op.
+"""
+from typing import List
+
+from ..base import Operator, Tensor
+from .toposort import toposort
+from .transform_utils import get_sorted_ops
+
+# ops whose generated launch code applies the accessor's offset and row pitch
+_GEMM_RCR_PREFIX = "gemm_rcr"
+_BMM_PREFIX = "bmm_"
+
+
+def _is_permute(name: str) -> bool:
+    return "permute" in name
+
+
+def _is_plain_gemm(name: str) -> bool:
+    return name.startswith(_GEMM_RCR_PREFIX) and not _is_permute(name)
+
+
+def _is_bmm(name: str) -> bool:
+    return (name.startswith(_BMM_PREFIX) or name.startswith("gemm_rrr")) and "softmax" not in name
+
+
+def can_read_strided(op: Operator, input_idx: int) -> bool:
+    """The op's launch code honours offset + pitch on input `input_idx`."""
+    name = op._attrs["op"]
+    if "input_accessors" not in op._attrs:
+        return False
+    if input_idx in (0, 1):  # A, B
+        return name.startswith(_GEMM_RCR_PREFIX) or _is_bmm(name)
+    if _is_plain_gemm(name):
+        # inputs are a, b, bias, d0, d1: the residuals may be views, the bias not
+        return input_idx >= 3
+    return False
+
+
+def can_write_strided(op: Operator) -> bool:
+    name = op._attrs["op"]
+    if "output_accessors" not in op._attrs or _is_permute(name):
+        return False
+    return _is_plain_gemm(name) or _is_bmm(name)
+
+
+def _rewire_split_piece(piece: Tensor, outputs: List[Tensor]) -> None:
+    x, dim, start = piece._attrs["strided_view_of"]
+    if piece._attrs["is_output"] or any(piece is o for o in outputs):
+        raise NotImplementedError(
+            f"a piece of a last-dim split ({piece._attrs['name']}) is a graph output: that needs a copy kernel, "
+            "which this backend does not have")
+    for op in list(piece.dst_ops()):
+        hit = [i for i, t in enumerate(op._attrs["inputs"]) if t is piece]
+        for i in hit:
+            if not can_read_strided(op, i):
+                raise NotImplementedError(
+                    f"op {op._attrs['op']} cannot read input {i} through an offset and a row pitch, which a piece "
+                    "of a last-dim split is; only GEMM-family operands and residuals can")
+            op._attrs["input_accessors"][i].update_base_tensor(x, dim, start)
+        op._attrs["inputs"] = [x if t is piece else t for t in op._attrs["inputs"]]
+        piece._attrs["dst_ops"].discard(op)
+        x._attrs["dst_ops"].add(op)
+
+
+def _fuse_splits(graph: List[Tensor], outputs: List[Tensor]) -> bool:
+    changed = False
+    for op in get_sorted_ops(graph):
+        if op._attrs["op"] != "split":
+            continue
+        pieces = [t for t in op._attrs["outputs"] if t._attrs.get("strided_view_of") is not None]
+        if not pieces:
+            continue
+        for piece in pieces:
+            _rewire_split_piece(piece, outputs)
+        # nothing reads the pieces any more: the split is unreachable from the outputs
+        op._attrs["inputs"][0]._attrs["dst_ops"].discard(op)
+        changed = True
+    return changed
+
+
+def _fuse_concats(graph: List[Tensor], outputs: List[Tensor]) -> bool:
+    changed = False
+    for cat in get_sorted_ops(graph):
+        if cat._attrs["op"] != "concatenate":
+            continue
+        out = cat._attrs["outputs"][0]
+        dim = cat._attrs["concat_dim"]
+        seen = set()
+        start = 0
+        out._attrs["src_ops"].discard(cat)
+        for t in cat._attrs["inputs"]:
+            producers = list(t.src_ops())
+            width = t._attrs["shape"][dim].value()
+            why = None
+            if id(t) in seen:
+                why = "appears twice in the concatenate"
+            elif len(producers) != 1 or not can_write_strided(producers[0]):
+                why = "is not written by a GEMM-family op that can write through an offset and a row pitch"
+            elif t._attrs["is_output"] or any(t is o for o in outputs):
+                why = "is a graph output as well"
+            elif len(list(t.dst_ops())) != 1:
+                why = "has other consumers"
+            elif t._attrs["is_view_of"] is not None:
+                why = "is a view"
+            if why is not None:
+                raise NotImplementedError(
+                    f"concatenate input {t._attrs['name']} {why}: that needs a copy kernel, which this backend "
+                    "does not have")
+            seen.add(id(t))
+            producer = producers[0]
+            producer._attrs["output_accessors"][0].update_base_tensor(out, dim, start)
+            producer._attrs["outputs"] = [out]
+            out._attrs["src_ops"].add(producer)
+            t._attrs["dst_ops"].discard(cat)
+            start += width
+        changed = True
+    return changed
+
+
+def fuse_strided_views(sorted_graph: List[Tensor], outputs: List[Tensor]) -> List[Tensor]:
+    """Apply both rewrites and return the re-sorted graph (unchanged object when nothing matched)."""
+    changed = _fuse_splits(sorted_graph, outputs)
+    changed = _fuse_concats(sorted_graph, outputs) or changed
+    return toposort(outputs) if changed else sorted_graph

@@ -65,6 +65,15 @@ def name_graph(sorted_graph: List[Tensor]) -> None:
             else:
                 d._attrs["name"] = valid_c_name(d._attrs["name"])
             dim_names.add(d._attrs["name"])
+    # dims that only an accessor still holds: the shape of a tensor that a split / concatenate fusion took out of
+    # the graph (the op reads or writes a view of a wider tensor, and its launcher is handed the view's dims)
+    for op in get_sorted_ops(sorted_graph):
+        for kind in ("input_accessors", "output_accessors"):
+            for k, acc in enumerate(op._attrs.get(kind) or []):
+                for i, d in enumerate(acc.original_shapes):
+                    if d._attrs["name"] is None:
+                        d._attrs["name"] = unique(f"{op._attrs['name']}_{kind[:-10]}{k}_dim_{i}")
+                    dim_names.add(d._attrs["name"])
     clash = dim_names & {t._attrs["name"] for t in sorted_graph}
     if clash:
         raise RuntimeError(f"dim names collide with tensor names: {sorted(clash)}")

@@ -392,6 +392,63 @@ def test_split_pieces_as_outputs_and_inputs():
     module.close()
 
 
+@pytest.mark.parametrize("Ms,K0,K1,N,dtype", [
+    ([16, 48], 96, 64, 40, "float16"),          # every offset and pitch a whole number of 16-byte pieces
+    ([300], 100, 60, 37, "float16"),            # odd offsets and pitches on A, C and the residual
+    ([1, 1000], 512, 256, 384, "bfloat16"),     # large tiles, a dynamic M down to one row
+])
+def test_last_dim_split_and_concatenate_around_gemms(Ms, K0, K1, N, dtype):
+    """Offset + row pitch on A, C and a residual, produced by the graph itself (the reference's
+    transform_strided_ops.py rewrites; its tests: tests/unittest/compiler/test_split_bmm_fusion.py,
+    test_strided_op_cat_pattern.py): two gemm_rcr_bias_add ops read the halves of a last-dim split of the
+    activations and of the residuals and write the halves of a concatenated output.  The rest of the output and the
+    neighbouring half of every operand must not leak into a result."""
+    print(f"case compile_model strided views Ms={Ms} K0={K0} K1={K1} N={N} {dtype}", flush=True)
+    tdt = {"float16": torch.float16, "bfloat16": torch.bfloat16}[dtype]
+    m = shape_utils.gen_int_var_min_max(Ms, name="m")
+    X = Tensor([m, IntImm(K0 + K1)], dtype=dtype, name="x", is_input=True)
+    R = Tensor([m, IntImm(2 * N)], dtype=dtype, name="r", is_input=True)
+    W0, B0 = Tensor([N, K0], dtype=dtype, name="w0", is_input=True), Tensor([N], dtype=dtype, name="b0", is_input=True)
+    W1, B1 = Tensor([N, K1], dtype=dtype, name="w1", is_input=True), Tensor([N], dtype=dtype, name="b1", is_input=True)
+    xa, xb = ops.split()(X, [K0, K1], dim=-1)
+    r0, r1 = ops.split()(R, N, dim=1)
+    y0 = ops.gemm_rcr_bias_add()(xa, W0, B0, r0)
+    y1 = ops.gemm_rcr_bias_add()(xb, W1, B1, r1)
+    Y = _mark_output(ops.concatenate()([y0, y1], dim=-1), "y")
+    module = compile_model(Y, detect_target(), WORKDIR, f"strided_views_{next(_counter)}")
+    for M in Ms:
+        x, r = _rand((M, K0 + K1), 1, dtype=tdt), _rand((M, 2 * N), 2, dtype=tdt)
+        w0, w1 = _rand((N, K0), 3, K0 ** -0.5, tdt), _rand((N, K1), 4, K1 ** -0.5, tdt)
+        b0, b1 = _rand((N,), 5, dtype=tdt), _rand((N,), 6, dtype=tdt)
+        want = torch.cat([
+            oracle.torch_gemm("gemm_rcr_bias_add", x[:, :K0].contiguous(), w0, b0, r[:, :N].contiguous()),
+            oracle.torch_gemm("gemm_rcr_bias_add", x[:, K0:].contiguous(), w1, b1, r[:, N:].contiguous())], dim=1)
+        y = torch.full((M, 2 * N), float("nan"), dtype=tdt, device="cuda")
+        module.run_with_tensors({"x": x.cuda(), "r": r.cuda(), "w0": w0.cuda(), "b0": b0.cuda(), "w1": w1.cuda(),
+                                 "b1": b1.cuda()}, [y])
+        torch.testing.assert_close(y.cpu().float(), want.to(tdt).float(), atol=1e-2, rtol=1e-2)
+    module.close()
+
+
+def test_last_dim_split_and_concatenate_around_batched_gemms():
+    """The same through the batched ops: bmm_rcr reads a piece of a 3-D tensor split along its last dim (batch
+    stride = rows x the wide pitch) and writes its columns of a concatenated 3-D output."""
+    print("case compile_model strided views bmm", flush=True)
+    B, M, N, K0, K1 = 5, 40, 24, 32, 16
+    X = Tensor([B, M, K0 + K1], name="x", is_input=True)
+    W0, W1 = Tensor([B, N, K0], name="w0", is_input=True), Tensor([B, N, K1], name="w1", is_input=True)
+    xa, xb = ops.split()(X, [K0, K1], dim=2)
+    Y = _mark_output(ops.concatenate()([ops.bmm_rcr()(xa, W0), ops.bmm_rcr()(xb, W1)], dim=2), "y")
+    module = compile_model(Y, detect_target(), WORKDIR, f"strided_views_bmm_{next(_counter)}")
+    x, w0, w1 = _rand((B, M, K0 + K1), 1), _rand((B, N, K0), 2, K0 ** -0.5), _rand((B, N, K1), 3, K1 ** -0.5)
+    want = torch.cat([oracle.torch_bmm_rcr(x[..., :K0].contiguous(), w0),
+                      oracle.torch_bmm_rcr(x[..., K0:].contiguous(), w1)], dim=2)
+    y = torch.full((B, M, 2 * N), float("nan"), dtype=torch.float16, device="cuda")
+    module.run_with_tensors({"x": x.cuda(), "w0": w0.cuda(), "w1": w1.cuda()}, [y])
+    torch.testing.assert_close(y.cpu().float(), want.half().float(), atol=1e-2, rtol=1e-2)
+    module.close()
+
+
 @pytest.mark.parametrize("B,S,D,H,qkv_bias,residual,causal", [
     (2, 384, 768, 12, True, True, False),      # BERT-base block shape
     (4, 197, 768, 12, True, True, False),      # ViT-B/16 block shape: sequence tail

@@ -569,8 +569,8 @@ def test_split_is_a_view_with_byte_offsets():
     assert [d.value() for d in b.shape()] == [1, 7, 4] and b._attrs["view_offset_bytes"] == 3 * 4 * 2
     parts = ops.split()(Tensor([10, 4], name="u", is_input=True), 4)  # torch semantics: 4, 4, 2
     assert [p.shape()[0].value() for p in parts] == [4, 4, 2]
-    with pytest.raises(NotImplementedError):
-        ops.split()(Tensor([2, 10], name="w", is_input=True), 5, dim=1)
+    with pytest.raises(NotImplementedError, match="middle dim"):
+        ops.split()(Tensor([2, 10, 4], name="w", is_input=True), 5, dim=1)
     with pytest.raises(RuntimeError, match="does not match"):
         ops.split()(Tensor([10, 4], name="t", is_input=True), [3, 3], dim=0)
     # offsets accumulate through views of views and reach the generated bindings
@@ -578,6 +578,112 @@ def test_split_is_a_view_with_byte_offsets():
 
     k2 = ops.reshape()(k, [-1, 8, 16])
     assert storage_offset_bytes(k2) == piece
+
+
+def _strided_view_graph(Ms=(48,), K0=96, K1=64, N=40):
+    """Two GEMMs between a last-dim split of the activations and of the residuals, and a concatenate."""
+    m = shape_utils.gen_int_var_min_max(list(Ms), name="m")
+    X = Tensor([m, IntImm(K0 + K1)], name="x", is_input=True)
+    R = Tensor([m, IntImm(2 * N)], name="r", is_input=True)
+    W0, B0 = Tensor([N, K0], name="w0", is_input=True), Tensor([N], name="b0", is_input=True)
+    W1, B1 = Tensor([N, K1], name="w1", is_input=True), Tensor([N], name="b1", is_input=True)
+    xa, xb = ops.split()(X, [K0, K1], dim=-1)
+    r0, r1 = ops.split()(R, N, dim=1)
+    y0 = ops.gemm_rcr_bias_add()(xa, W0, B0, r0)
+    y1 = ops.gemm_rcr_bias_add()(xb, W1, B1, r1)
+    Y = ops.concatenate()([y0, y1], dim=-1)
+    Y._attrs["name"] = "y"
+    Y._attrs["is_output"] = True
+    return Y, (xa, xb, r0, r1, y0, y1)
+
+
+def test_last_dim_split_and_concatenate_become_offsets_and_pitches(tmp_path, monkeypatch):
+    """The rewrites of the reference's transform_strided_ops.py:33-64 on the GEMM family: pieces of a last-dim split
+    are read, and inputs of a last-dim concatenate are written, through TensorAccessor.update_base_tensor."""
+    K0, K1, N = 96, 64, 40
+    Y, (xa, xb, r0, r1, y0, y1) = _strided_view_graph(K0=K0, K1=K1, N=N)
+    assert xb._attrs["strided_view_of"][1:] == (1, K0) and "view_offset_bytes" not in xb._attrs
+    graph = transform.toposort(Y)
+    assert {op._attrs["op"] for op in transform.get_sorted_ops(graph)} == {"split", "gemm_rcr_bias_add", "concatenate"}
+    graph = transform.fuse_strided_views(graph, [Y])
+    sorted_ops = transform.get_sorted_ops(graph)
+    assert [op._attrs["op"] for op in sorted_ops] == ["gemm_rcr_bias_add"] * 2
+    assert all(t not in graph for t in (xa, xb, r0, r1, y0, y1))
+    g0, g1 = sorted_ops
+    assert [t._attrs["name"] for t in g1._attrs["inputs"]] == ["x", "w1", "b1", "r"] and g1._attrs["outputs"] == [Y]
+    a, _, _, d = g1._attrs["input_accessors"]
+    c = g1._attrs["output_accessors"][0]
+    assert (a.offset, a.row_pitch(), a.is_contiguous) == (K0, K0 + K1, False)
+    assert [x.value() for x in a.original_shapes[1:]] == [K1]
+    assert (d.offset, d.row_pitch()) == (N, 2 * N) and (c.offset, c.row_pitch()) == (N, 2 * N)
+    assert g0._attrs["input_accessors"][0].offset == 0 and g0._attrs["output_accessors"][0].row_pitch() == 2 * N
+    assert list(Y.src_ops()) == [g0, g1]
+    # the problem sizes still come from the views' own shapes
+    g1._extract_exec_path(DynamicProfileStrategy.MAX)
+    assert list(g1._attrs["exec_path"]) == [f"M == 48 && N == {N} && K == {K1}"]
+
+    # through compile_model: generated launch code and the dim members of the vanished views
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    reset_name_counters()
+    Y, _ = _strided_view_graph(Ms=(16, 48), K0=K0, K1=K1, N=N)
+    import torch
+
+    if torch.cuda.is_available():
+        compile_model(Y, detect_target(), str(tmp_path), "strided").close()
+    else:
+        with pytest.raises(RuntimeError, match="AITemplateModelContainerCreate"):
+            compile_model(Y, detect_target(), str(tmp_path), "strided")
+    build = tmp_path / "strided"
+    model_src = (build / "model-generated.cpp").read_text()
+    entries = re.findall(r'OpEntry\{"(\w+)"', model_src)
+    assert len(entries) == 2
+    srcs = [(build / f"{e}.cpp").read_text() for e in entries]
+    assert f"static_cast<const uint16_t*>(in_ptr) + {K0};" in srcs[1] and f"const int64_t lda = {K0 + K1};" in srcs[1]
+    assert f"static_cast<uint16_t*>(out_ptr) + {N};" in srcs[1] and f"const int64_t ldc = {2 * N};" in srcs[1]
+    assert f"const uint16_t* d0 = static_cast<const uint16_t*>(d0_ptr) + {N};" in srcs[1]
+    assert f"const int64_t ldd = {2 * N};" in srcs[1] and "bias_ptr, d0, nullptr, c, M, N, K" in srcs[1]
+    assert "static_cast<const uint16_t*>(in_ptr) + 0;" in srcs[0] and f"const int64_t lda = {K0 + K1};" in srcs[0]
+    # both ops are handed x, r and y; the views' static dims are members of the model
+    assert model_src.count("(x, w") == 2 and model_src.count(", y, b") == 2
+    for e in entries:
+        assert re.search(rf"int64_t {e}_input0_dim_1 \{{({K0}|{K1})\}};", model_src), e
+        assert f"&m, &{e}_input0_dim_1" in model_src
+
+
+def test_strided_views_that_need_a_copy_kernel_are_refused():
+    N, K = 16, 32
+    X = Tensor([8, 2 * K], name="x", is_input=True)
+    W, B = Tensor([N, K], name="w", is_input=True), Tensor([N], name="b", is_input=True)
+    xa, xb = ops.split()(X, K, dim=1)
+    # a piece read by an op without accessors, a piece that is an output
+    out = ops.reshape()(xb, [4, -1])
+    out._attrs["is_output"] = True
+    with pytest.raises(NotImplementedError, match="cannot read input 0 through an offset"):
+        transform.fuse_strided_views(transform.toposort(out), [out])
+    xa, xb = ops.split()(X, K, dim=1)
+    xa._attrs["is_output"] = True
+    with pytest.raises(NotImplementedError, match="graph output"):
+        transform.fuse_strided_views(transform.toposort(xa), [xa])
+    # a bias cannot be a view
+    b0, b1 = ops.split()(Tensor([1, 2 * N], name="b2", is_input=True), N, dim=1)
+    # (dims of size 1 in front: this is the contiguous kind of split, not a strided view)
+    assert "strided_view_of" not in b1._attrs
+    # concatenate of a graph input, of a tensor with a second consumer, along another dim
+    y = ops.gemm_rcr_bias()(X, Tensor([N, 2 * K], name="w2", is_input=True), B)
+    cat = ops.concatenate()([y, Tensor([8, N], name="z", is_input=True)], dim=1)
+    cat._attrs["is_output"] = True
+    with pytest.raises(NotImplementedError, match="is not written by a GEMM-family op"):
+        transform.fuse_strided_views(transform.toposort(cat), [cat])
+    y = ops.gemm_rcr_bias()(X, Tensor([N, 2 * K], name="w3", is_input=True), B)
+    y2 = ops.gemm_rcr_bias()(y, Tensor([N, N], name="w4", is_input=True), B)
+    cat = ops.concatenate()([y, y2], dim=-1)
+    cat._attrs["is_output"] = True
+    with pytest.raises(NotImplementedError, match="has other consumers"):
+        transform.fuse_strided_views(transform.toposort(cat), [cat])
+    with pytest.raises(NotImplementedError, match="other than the last"):
+        ops.concatenate()([y, y2], dim=0)
+    with pytest.raises(RuntimeError, match="dim 0 differs"):
+        ops.concatenate()([y, Tensor([9, N], name="z2", is_input=True)], dim=1)
 
 
 def test_multihead_attention_block_compiles_to_three_kernels(tmp_path, monkeypatch):
