@@ -44,11 +44,11 @@ template <class Tile, bool PERM, int LAYOUT>
 struct KernelOf {
   static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi, PERM, LAYOUT>;
 };
-template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, int SPLITK, bool PERM,
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, int MODE, bool PERM,
           int LAYOUT>
-struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, SPLITK>, PERM, LAYOUT> {
+struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>, PERM, LAYOUT> {
   static constexpr auto value =
-      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, SPLITK>, Epi, PERM, LAYOUT>;
+      gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>, Epi, PERM, LAYOUT>;
 };
 
 template <int BM, int BN, int BK, int WM, int WN, int NS, bool PERM, int LAYOUT>
@@ -247,9 +247,18 @@ const GemmAlgo kAlgos[] = {
                   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>::kLdsBytes),                      \
    4, 1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>>,                             \
    &workspace_of<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 1>>},
+#define AITAMD_GEMM_TILE_DMA_K2(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT)                                      \
+  {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
+   "_k2",                                                                                                 \
+   BM, BN, BK, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>::NT, 2,                             \
+   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>::kLdsBytes,                                     \
+   dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>::NT, OCC,                        \
+                  GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>::kLdsBytes),                      \
+   1, 1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>>, nullptr},
 #include "gemm_tiles.inc"
 #undef AITAMD_GEMM_TILE
 #undef AITAMD_GEMM_TILE_DMA
+#undef AITAMD_GEMM_TILE_DMA_K2
 #undef AITAMD_GEMM_TILE_PERSIST
 #undef AITAMD_GEMM_TILE_DMA_SPLITK
 };

@@ -300,12 +300,14 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;
     const T* bias = reinterpret_cast<const T*>(p.bias);
 
-    bool vec_ok = ((p.N & 3) == 0) && ((p.ldc & 3) == 0) && ((p.sc & 3) == 0) && (!PERM || (p.perm_n2 & 3) == 0) &&
-        ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
-    if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 7) == 0);
+    // vector form for the lanes whose 4 columns lie inside the row: multi-dword global and buffer accesses need
+    // dword alignment only, so even pitches and 4-byte aligned pointers are enough
+    bool vec_ok = ((p.ldc & 1) == 0) && ((p.sc & 1) == 0) && (!PERM || ((p.perm_n2 & 3) == 0 && (p.N & 3) == 0)) &&
+        ((reinterpret_cast<uintptr_t>(p.c) & 3) == 0);
+    if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 3) == 0);
     if (Epi::kNumD >= 1)
-      vec_ok = vec_ok && ((p.ldd & 3) == 0) && ((p.sd & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 7) == 0);
-    if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 7) == 0);
+      vec_ok = vec_ok && ((p.ldd & 1) == 0) && ((p.sd & 1) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 3) == 0);
+    if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 3) == 0);
 
     using vec4 = typename Tr::vec4;
 #pragma unroll
@@ -323,7 +325,7 @@ __global__ void __launch_bounds__(Tile::NT) gemm_rcr_kernel(const GemmParams p) 
           for (int j = 0; j < 4; ++j) v[j] = acc[mi][ni][g * 4 + j];
           const int64_t c_idx = out_index<PERM>(p, m, n);
           const int64_t d_idx = (int64_t)m * p.ldd + n;
-          if (vec_ok) {
+          if (vec_ok && n + 4 <= p.N) {
             vec4 bv = {}, d0v = {}, d1v = {};
             if constexpr (Epi::kHasBias) bv = *reinterpret_cast<const vec4*>(bias + n);
             if constexpr (Epi::kNumD >= 1) d0v = *reinterpret_cast<const vec4*>(D0b + d_idx);

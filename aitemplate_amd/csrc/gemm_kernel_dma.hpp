@@ -25,10 +25,17 @@ namespace aitamd {
 // tile's counter, and the one that finds all the others counted sums the partial tiles in slab order (its own
 // included, so the result does not depend on who came last) and runs the epilogue.  Nobody waits for anybody.
 // For grids that leave most CUs idle and tiles small enough that a partial tile is a few KiB.
+//
+// MODE 2, K in dwords: K, the row pitches and the operand pointers need to be whole dwords only (K % 8 in {2, 4, 6}:
+// rows that start 4, 8 or 12 bytes off a 16-byte boundary).  The 16-byte slab loads take dword-aligned addresses
+// as they are; the K loop runs over the whole 16-byte pieces of a row, and the 2, 4 or 6 elements behind them are
+// fetched once per tile with dword loads straight into MFMA operands (lanes of the first k-chunk, zeros elsewhere)
+// and multiplied after the loop.  Nothing is read past the end of a row.
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int OCC_, int PIPE_ = 0, int MT_ = 32, int AUX_ = 0,
-          int SPLITK_ = 0>
+          int MODE_ = 0>
 struct GemmTileDma {
-  static constexpr int SPLITK = SPLITK_;
+  static constexpr int SPLITK = MODE_ == 1;
+  static constexpr int KTAIL = MODE_ == 2;
   static constexpr int64_t kSlotBytes = (int64_t)BM_ * BN_ * 4;
   static constexpr int64_t kCounterAlign = 4096;
   // scratch bytes for `tiles` (batch x tile) pairs shared by `splits` workgroups each: one counter per pair,
@@ -48,7 +55,7 @@ struct GemmTileDma {
   static constexpr int ACC_N = MT * MT / 64;         // fp32 accumulators per lane per MFMA tile
   static constexpr int BM = BM_, BN = BN_, BK = BK_;
   static constexpr int WGM = WGM_, WGN = WGN_, NS = NS_, OCC = OCC_;
-  static constexpr int KVEC = 8;
+  static constexpr int KVEC = KTAIL ? 2 : 8;
   static constexpr int NW = WGM * WGN;
   static constexpr int NT = NW * kWaveSize;
   static constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -254,7 +261,10 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
           (fq * 8 + (t_r >> 2)) * BN;
   }
 
-  const int k_tiles_all = (p.K + BK - 1) / BK;
+  static_assert(!Tile::KTAIL || LAYOUT == 0, "the dword K tail is written for K-contiguous operands");
+  // K covered by the slab loop: all of it, or its whole 16-byte pieces
+  const int k_main = Tile::KTAIL ? (p.K & ~7) : p.K;
+  const int k_tiles_all = (k_main + BK - 1) / BK;
   // this workgroup's K-slabs [k_lo, k_lo + k_tiles)
   const int splits = Tile::SPLITK ? p.split_k : 1;
   const int k_lo = Tile::SPLITK ? (int)((int64_t)split * k_tiles_all / splits) : 0;
@@ -273,14 +283,14 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     // the end of K are still issued (every chunk out of range -> zero fill) so
     // the number of loads in flight per step stays constant for s_waitcnt.
     auto issue_loads = [&](int kt, int stage, int i0, int i1) {
-      const int k0 = (Tile::SPLITK && kt >= k_tiles) ? p.K : (k_lo + kt) * BK;  // (past the own range: nothing to fetch)
+      const int k0 = (Tile::SPLITK && kt >= k_tiles) ? k_main : (k_lo + kt) * BK;  // (past the own range: nothing to fetch)
       T* sbase = smem + stage * Tile::STAGE_ELEMS;
 #pragma unroll
       for (int i = 0; i < L_IT; ++i) {
         if (i < i0 || i >= i1) continue;
         const int j = wave + i * Tile::NW;
         const uint32_t step = (A_T || B_T) ? (uint32_t)k0 * l_kbytes[i] : (uint32_t)(k0 * 2);
-        const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + step : kOobOffset;
+        const uint32_t off = (k0 + l_chunk_k[i] < k_main) ? l_off[i] + step : kOobOffset;
         T* dst = sbase + j * 512;  // 1 KiB = 512 elements per wave-load; A blocks then B blocks
         const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
         if (is_a)
@@ -298,6 +308,27 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
       for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
         for (int e = 0; e < ACC_N; ++e) acc[mi][ni][e] = 0.0f;
+
+    // dword K tail: the up to three dwords behind the last whole 16-byte piece of each of the lane's operand rows,
+    // requested before the slab loads (so every wait of the loop covers them) and used after the loop
+    uint32_t tail_a[Tile::KTAIL ? MI : 1][3], tail_b[Tile::KTAIL ? NI : 1][3];
+    if constexpr (Tile::KTAIL != 0) {
+#pragma unroll
+      for (int d = 0; d < 3; ++d) {
+        const int k = k_main + 2 * d;
+        const bool on = fq == 0 && k < p.K;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+          const int row = wm * Tile::WTM + mi * MT + fr;
+          tail_a[mi][d] = buffer_load_4B(ra, on ? (uint32_t)(((int64_t)row * p.lda + k) * 2) : kOobOffset);
+        }
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+          const int row = wn * Tile::WTN + ni * MT + fr;
+          tail_b[ni][d] = buffer_load_4B(rb, on ? (uint32_t)(((int64_t)row * p.ldb + k) * 2) : kOobOffset);
+        }
+      }
+    }
 
     // the L_IT wave-loads of a slab are issued in KK equal portions, one per MFMA step
     constexpr int L_PER = (L_IT + KK - 1) / KK;
@@ -407,6 +438,18 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     // drain the zero-fill slabs still in flight before LDS is reused
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
+    if constexpr (Tile::KTAIL != 0) {
+      if (k_main < p.K) {
+        vec8 ta[MI], tb[NI];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+          ta[mi] = __builtin_bit_cast(vec8, u32x4{tail_a[mi][0], tail_a[mi][1], tail_a[mi][2], 0u});
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+          tb[ni] = __builtin_bit_cast(vec8, u32x4{tail_b[ni][0], tail_b[ni][1], tail_b[ni][2], 0u});
+        mfmas(ta, tb);
+      }
+    }
 
     if constexpr (Tile::SPLITK != 0) {
       // ---------------- split-K: partial tile to the scratch memory; the last workgroup of the tile sums ----
@@ -484,12 +527,14 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     const T* D1b = Epi::kNumD >= 2 ? reinterpret_cast<const T*>(p.d1) + (int64_t)batch * p.sd : nullptr;
     const T* bias = reinterpret_cast<const T*>(p.bias);
 
-    bool vec_ok = ((p.N & 7) == 0) && ((p.ldc & 7) == 0) && ((p.sc & 7) == 0) && (!PERM || (p.perm_n2 & 7) == 0) &&
-        ((reinterpret_cast<uintptr_t>(p.c) & 15) == 0);
-    if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
+    // vector form for the lanes whose 8 columns lie inside the row: multi-dword global and buffer accesses need
+    // dword alignment only, so even pitches and 4-byte aligned pointers are enough
+    bool vec_ok = ((p.ldc & 1) == 0) && ((p.sc & 1) == 0) && (!PERM || ((p.perm_n2 & 7) == 0 && (p.N & 7) == 0)) &&
+        ((reinterpret_cast<uintptr_t>(p.c) & 3) == 0);
+    if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 3) == 0);
     if (Epi::kNumD >= 1)
-      vec_ok = vec_ok && ((p.ldd & 7) == 0) && ((p.sd & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 15) == 0);
-    if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 15) == 0);
+      vec_ok = vec_ok && ((p.ldd & 1) == 0) && ((p.sd & 1) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 3) == 0);
+    if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 3) == 0);
 
     constexpr int PITCH = Tile::EPI_PITCH;
     float* strip = reinterpret_cast<float*>(smem_raw) + wave * MT * PITCH;
@@ -529,7 +574,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
           float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
           const int64_t c_idx = out_index<PERM>(p, m, n);
           const int64_t d_idx = (int64_t)m * p.ldd + n;
-          if (vec_ok) {
+          if (vec_ok && n + 8 <= p.N) {
             vec8 bv = {}, d0v = {}, d1v = {};
             if constexpr (Epi::kHasBias) bv = *reinterpret_cast<const vec8*>(bias + n);
             if constexpr (Epi::kNumD >= 1) d0v = *reinterpret_cast<const vec8*>(D0b + d_idx);

@@ -23,9 +23,6 @@
 
 #include "gemm_kernel_dma.hpp"
 
-#ifndef TILE_STAMP
-#define TILE_STAMP(i, k)
-#endif
 
 namespace aitamd {
 
@@ -216,23 +213,25 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   // ---- epilogue -------------------------------------------------------------------------------
   const T* bias = reinterpret_cast<const T*>(p.bias);
-  bool vec_ok = ((p.N & 7) == 0) && ((p.ldc & 7) == 0) && ((p.sc & 7) == 0) && (!PERM || (p.perm_n2 & 7) == 0) &&
-      ((reinterpret_cast<uintptr_t>(p.c) & 15) == 0);
-  if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
+  // vector form for the lanes whose 8 columns lie inside the row: multi-dword global and buffer accesses need
+  // dword alignment only, so even pitches and 4-byte aligned pointers are enough
+  bool vec_ok = ((p.ldc & 1) == 0) && ((p.sc & 1) == 0) && (!PERM || ((p.perm_n2 & 7) == 0 && (p.N & 7) == 0)) &&
+      ((reinterpret_cast<uintptr_t>(p.c) & 3) == 0);
+  if (Epi::kHasBias) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.bias) & 3) == 0);
   if (Epi::kNumD >= 1)
-    vec_ok = vec_ok && ((p.ldd & 7) == 0) && ((p.sd & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 15) == 0);
-  if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 15) == 0);
+    vec_ok = vec_ok && ((p.ldd & 1) == 0) && ((p.sd & 1) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 3) == 0);
+  if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 3) == 0);
   // strip addressing: row r, 16-byte chunk c lives at r * PITCH + ((c ^ (r % SC)) << 4)
   const int w_base = fr * Tile::STRIP_PITCH + fq * 8;
   const int w_swz = fr & (SC - 1);
   const int r_row = lane / SC;
   const int r_c = lane % SC;
 
-  // Fast form of the epilogue's addressing (plain store, everything 16-byte aligned, a tile's rows span less than
+  // Fast form of the epilogue's addressing (plain store, N a multiple of 8, a tile's rows span less than
   // 2 GiB): the output and the residuals are addressed through buffer descriptors that start at the wave's
   // corner of the tile, with 32-bit byte offsets that advance by a scalar per 8-row pass - no 64-bit index
   // arithmetic per pass, rows past M cut off by the descriptor's size, columns past N by an out-of-range offset.
-  const bool fast_addr = !PERM && vec_ok && (int64_t)BM * p.ldc * 2 < 0x7fffffffll &&
+  const bool fast_addr = !PERM && vec_ok && (p.N & 7) == 0 && (int64_t)BM * p.ldc * 2 < 0x7fffffffll &&
       (Epi::kNumD == 0 || (int64_t)BM * p.ldd * 2 < 0x7fffffffll);
   const uint32_t lane_off_c = (uint32_t)((r_row * (int)p.ldc + r_c * 8) * 2);
   const uint32_t lane_off_d = (uint32_t)((r_row * (int)p.ldd + r_c * 8) * 2);
@@ -325,7 +324,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     const int n = c.n0 + wn * Tile::WTN + r_c * 8;  // the lane's 8 columns: the same in every pass
     float bf8[8] = {};  // the lane's 8 bias values, converted once per tile
     if constexpr (Epi::kHasBias) {
-      if (vec_ok && n < p.N) {
+      if (vec_ok && n + 8 <= p.N) {
         const vec8 bv = *reinterpret_cast<const vec8*>(bias + n);
 #pragma unroll
         for (int j = 0; j < 8; ++j) bf8[j] = Tr::to_float(bv[j]);
@@ -355,7 +354,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         if (m < p.M && n < p.N) {
           const int64_t c_idx = out_index<PERM>(p, m, n);
           const int64_t d_idx = (int64_t)m * p.ldd + n;
-          if (vec_ok) {
+          if (vec_ok && n + 8 <= p.N) {
             vec8 d0v = {}, d1v = {};
             if constexpr (Epi::kNumD >= 1) d0v = *reinterpret_cast<const vec8*>(D0b + d_idx);
             if constexpr (Epi::kNumD >= 2) d1v = *reinterpret_cast<const vec8*>(D1b + d_idx);
@@ -398,7 +397,6 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     // waves whose rows lie outside a half tile keep the ring turning (their share of the loads, the
     // waits and the barriers) but multiply and store nothing; a half tile is always the last item
     const bool active = wm * Tile::WTM < cur.rows;
-    TILE_STAMP(i, 0);
     for (int kt = 0; kt < k_tiles; ++kt) {
       const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
       const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
@@ -429,9 +427,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       }
       rd_stage = nx_stage;
     }
-    TILE_STAMP(i, 1);
     if (active) epilogue(cur);
-    TILE_STAMP(i, 2);
   }
   // no LDS-DMA may be in flight into a workgroup that has ended
   wait_vmcnt<0>();

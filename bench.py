@@ -7,8 +7,11 @@ input that is already resident in HBM.  Operand sets rotate through a pool large
 
 Prints ONE JSON line:  value = TFLOP/s over the K timed steps (wall clock between two device
 synchronisations);  roofline.achieved = algorithmic FLOPs / average launch duration from HIP
-events recorded around the same K launches on the launch stream;  cpu_baseline = the
-reference tests' PyTorch fp32 expression timed on the host cores.
+events recorded around the same K launches on the launch stream (events at group boundaries
+inside the same region give the median of the per-group averages beside it);
+other_configs = the remaining benchmark configurations, each on the instance an untimed
+profiling pass picked, each with its own roofline;  cpu_baseline = the reference tests'
+PyTorch fp32 expression timed on the host cores.
 """
 import argparse
 import json
@@ -23,14 +26,12 @@ if ROOT not in sys.path:
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the headline workload, per kernel instance, from two counter runs of
-# this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter read for the
-# 256 MiB copy of --copy-probe in the same run.  Instances never measured report null.
-MEASURED_TRAFFIC_BYTES = {
-    # scale factors from a 256 MiB device copy in the same run: it reads 131084.7 KiB by FETCH_SIZE (x 2.000)
-    # and writes 262144 KiB by WRITE_SIZE (x 1.000)
-    # FETCH_SIZE 88089.3 KiB x 2.000 + WRITE_SIZE 147456.3 KiB x 1.000 (with streaming output stores)
-    "gemm_rcr_f16_256x256x32_w2x4_persist4": 331_402_000,
+# HBM bytes per launch of the headline workload, per kernel instance: (bytes, the file under profiles/ that holds
+# the two counter runs of this script the figure comes from: FETCH_SIZE, then WRITE_SIZE, each scaled by what the
+# same counter read for the 256 MiB copy of --copy-probe in the same run).  An instance that is not listed was
+# never measured and reports null with that reason.
+MEASURED_TRAFFIC = {
+    "gemm_rcr_f16_256x256x32_w2x4_persist4": (331_402_000, "profiles/gemm_rcr_bias_gelu_c2a_hbm_traffic.txt"),
 }
 
 SHAPES = {
@@ -40,6 +41,55 @@ SHAPES = {
     "c2b": ("gemm_rcr_bias_add", 24576, 768, 3072, 1),
     "c3": ("gemm_rcr_bias_add_add", 12608, 1024, 4096, 2),
 }
+
+
+def _median(values):
+    v = sorted(values)
+    n = len(v)
+    return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
+
+
+def timed_region(torch, step, steps, warmup, groups=20, graph=False):
+    """W untimed steps, then exactly K steps between two device synchronisations.  Events on the launch stream
+    bracket the region and cut it into up to `groups` groups of consecutive launches: the region's average and
+    the median of the group averages both come from the same K launches.  With `graph` the K steps are captured
+    once (untimed) and the timed region replays them: for kernels of a few microseconds, whose launches the host
+    cannot issue as fast as the GPU retires them."""
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    groups = max(1, min(groups, steps))
+    cuts = [steps * g // groups for g in range(groups + 1)]
+    if graph:
+        per = steps // groups or 1
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()  # default priority
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                for i in range(per):
+                    step(i)
+        torch.cuda.current_stream().wait_stream(side)
+        g.replay()  # untimed: the first replay uploads the graph
+        torch.cuda.synchronize()
+        cuts = [per * k for k in range(groups + 1)]
+        steps = per * groups
+    events = [torch.cuda.Event(enable_timing=True) for _ in cuts]
+    t0 = time.perf_counter()
+    events[0].record()
+    for k in range(groups):
+        if graph:
+            g.replay()
+        else:
+            for i in range(cuts[k], cuts[k + 1]):
+                step(i)
+        events[k + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per_group = [events[k].elapsed_time(events[k + 1]) / (cuts[k + 1] - cuts[k]) for k in range(groups)]
+    return {"steps": steps, "wall_ms_per_step": wall_ms / steps,
+            "event_ms_per_launch": events[0].elapsed_time(events[-1]) / steps,
+            "median_ms_per_launch": _median(per_group), "groups": groups}
 
 
 def _make_pool(torch, op, M, N, K, nres, pool_bytes=600 << 20):
@@ -57,78 +107,90 @@ def _make_pool(torch, op, M, N, K, nres, pool_bytes=600 << 20):
     return pool
 
 
-def time_gemm(torch, eager, name, steps, warmup, algo=-1):
-    op, M, N, K, nres = SHAPES[name]
-    pool = _make_pool(torch, op, M, N, K, nres)
+class GemmCase:
+    """One GEMM configuration: its operand pool and, for the instances that split K, the scratch memory."""
 
-    def step(i):
-        x, w, b, d, out = pool[i % len(pool)]
-        eager.gemm(op, x, w, b, d[0] if nres >= 1 else None, d[1] if nres >= 2 else None, out=out, algo=algo)
+    def __init__(self, torch, eager, kernels, name):
+        self.torch, self.eager, self.kernels, self.name = torch, eager, kernels, name
+        self.op, self.M, self.N, self.K, self.nres = SHAPES[name]
+        self.epi = kernels.EPILOGUE_OF_OP[self.op]
+        self.pool = _make_pool(torch, self.op, self.M, self.N, self.K, self.nres)
+        lib = kernels.load()
+        self.supported = [a for a in range(lib.aitamd_gemm_num_algos(self.epi, 0))
+                          if lib.aitamd_gemm_algo_supported(self.epi, 0, a, self.M, self.N, self.K, self.K, self.K, 16)]
+        need = max([eager.gemm_workspace_bytes(self.op, a, self.M, self.N, self.K) for a in self.supported] + [0])
+        self.workspace = eager.new_workspace(need) if need > 0 else None
+        self.flops = 2 * self.M * self.N * self.K
+        self.bytes = 2 * (self.M * self.K + self.N * self.K + self.N + (1 + self.nres) * self.M * self.N)
 
-    for i in range(warmup):
-        step(i)
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        step(i)
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ev_ms = e0.elapsed_time(e1)
-    return {"wall_ms_per_step": wall_ms / steps, "event_ms_per_launch": ev_ms / steps,
-            "flops": 2 * M * N * K, "bytes": 2 * (M * K + N * K + N + (1 + nres) * M * N)}
+    def step_fn(self, algo):
+        pool, op, nres, ws, gemm = self.pool, self.op, self.nres, self.workspace, self.eager.gemm
+
+        def step(i):
+            x, w, b, d, out = pool[i % len(pool)]
+            gemm(op, x, w, b, d[0] if nres >= 1 else None, d[1] if nres >= 2 else None, out=out, algo=algo,
+                 workspace=ws)
+        return step
+
+    def pick_instance(self, iters=15):
+        """Untimed selection pass, the same procedure compile_model's profiling step applies
+        (python/aitemplate/compiler/ops/gemm_universal/gemm_common.py:743-829 in the reference):
+        time every instance that supports the problem and keep the fastest."""
+        best, best_ms = -1, float("inf")
+        for algo in self.supported:
+            ms = timed_region(self.torch, self.step_fn(algo), iters, 3, groups=1)["event_ms_per_launch"]
+            if ms < best_ms:
+                best, best_ms = algo, ms
+        return best
+
+    def instance_name(self, algo):
+        return self.kernels.gemm_algo_names(self.epi, 0)[algo]
 
 
-def time_call(torch, fn, steps, warmup):
-    for i in range(warmup):
-        fn(i)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(steps):
-        fn(i)
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps
+def _roofline(bound, work, ms_avg, ms_median):
+    """work = algorithmic FLOPs (bound "mfma") or bytes (bound "hbm") of one launch."""
+    peak, unit, scale = (PEAK_FP16_TFLOPS, "TFLOP/s", 1e9) if bound == "mfma" else (PEAK_HBM_GBS, "GB/s", 1e6)
+    achieved = work / ms_avg / scale
+    return {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "frac_at_median_launch": round(work / ms_median / scale / peak, 4)}
 
 
-def time_c4_c5(torch, eager, steps, warmup):
-    """bmm_rcr (config 4, against the HBM roofline) and bmm_softmax_bmm_permute (config 5)."""
+def other_configs(torch, eager, kernels, steps, warmup):
+    """Configurations 1, 2b, 3 (MFMA-bound GEMMs), 4 (bmm_rcr, HBM-bound) and 5 (fused attention)."""
+    out = {}
+    for name in ("c1", "c2b", "c3"):
+        case = GemmCase(torch, eager, kernels, name)
+        algo = case.pick_instance()
+        # a launch of config 1 lasts a few microseconds: replay a captured graph so the GPU, not the host, sets the pace
+        graph = name == "c1"
+        r = timed_region(torch, case.step_fn(algo), steps, warmup, graph=graph)
+        ws = eager.gemm_workspace_bytes(case.op, algo, case.M, case.N, case.K)
+        out[name] = {"op": case.op, "M": case.M, "N": case.N, "K": case.K, "instance": case.instance_name(algo),
+                     "workspace_bytes": ws, "launches": "graph replay" if graph else "direct",
+                     "ms": round(r["event_ms_per_launch"], 5), "median_ms": round(r["median_ms_per_launch"], 5),
+                     "tflops": round(case.flops / r["event_ms_per_launch"] / 1e9, 2),
+                     "roofline": _roofline("mfma", case.flops, r["event_ms_per_launch"], r["median_ms_per_launch"])}
+        del case
     g = torch.Generator(device="cuda").manual_seed(4)
     sets4 = [(torch.randn(768, 384, 64, device="cuda", generator=g).half() / 8,
               torch.randn(768, 384, 64, device="cuda", generator=g).half() / 8,
               torch.empty(768, 384, 384, device="cuda", dtype=torch.float16)) for _ in range(3)]
-    ms4 = time_call(torch, lambda i: eager.bmm_rcr(sets4[i % 3][0], sets4[i % 3][1], out=sets4[i % 3][2]), steps, warmup)
+    r4 = timed_region(torch, lambda i: eager.bmm_rcr(sets4[i % 3][0], sets4[i % 3][1], out=sets4[i % 3][2]), steps, warmup)
     b4 = 2 * 768 * (2 * 384 * 64 + 384 * 384)
+    out["c4"] = {"op": "bmm_rcr", "B": 768, "M": 384, "N": 384, "K": 64, "ms": round(r4["event_ms_per_launch"], 5),
+                 "median_ms": round(r4["median_ms_per_launch"], 5),
+                 "roofline": _roofline("hbm", b4, r4["event_ms_per_launch"], r4["median_ms_per_launch"])}
+    del sets4
     sets5 = [tuple(torch.randn(16, 4096, 40, device="cuda", generator=g).half() for _ in range(3)) for _ in range(16)]
     out5 = torch.empty(2, 4096, 8, 40, device="cuda", dtype=torch.float16)
-    ms5 = time_call(torch, lambda i: eager.bmm_softmax_bmm_permute(*sets5[i % 16], shape=(8,), scale=40 ** -0.5, out=out5),
-                    steps, warmup)
+    r5 = timed_region(torch, lambda i: eager.bmm_softmax_bmm_permute(*sets5[i % 16], shape=(8,), scale=40 ** -0.5, out=out5),
+                      steps, warmup)
     f5 = 4 * 16 * 4096 * 4096 * 40
-    return {"c4": {"op": "bmm_rcr", "ms": round(ms4, 5), "gbs": round(b4 / ms4 / 1e6, 1),
-                   "frac_of_hbm_peak": round(b4 / ms4 / 1e6 / PEAK_HBM_GBS, 4)},
-            "c5": {"op": "bmm_softmax_bmm_permute", "ms": round(ms5, 5), "tflops": round(f5 / ms5 / 1e9, 2),
-                   "frac_of_mfma_peak": round(f5 / ms5 / 1e9 / PEAK_FP16_TFLOPS, 4)}}
-
-
-def pick_instance(torch, eager, kernels, name, iters=15):
-    """Untimed selection pass, the same procedure compile_model's profiling step applies
-    (python/aitemplate/compiler/ops/gemm_universal/gemm_common.py:743-829 in the reference):
-    time every instance that supports the problem and keep the fastest."""
-    op, M, N, K, nres = SHAPES[name]
-    epi = kernels.EPILOGUE_OF_OP[op]
-    lib = kernels.load()
-    best, best_ms = -1, float("inf")
-    for algo in range(lib.aitamd_gemm_num_algos(epi, 0)):
-        if not lib.aitamd_gemm_algo_supported(epi, 0, algo, M, N, K, K, K, 16):
-            continue
-        ms = time_gemm(torch, eager, name, iters, 3, algo)["event_ms_per_launch"]
-        if ms < best_ms:
-            best, best_ms = algo, ms
-    return best
+    out["c5"] = {"op": "bmm_softmax_bmm_permute", "B": 16, "M": 4096, "N": 4096, "K": 40, "O": 40,
+                 "ms": round(r5["event_ms_per_launch"], 5), "median_ms": round(r5["median_ms_per_launch"], 5),
+                 "tflops": round(f5 / r5["event_ms_per_launch"] / 1e9, 2),
+                 "roofline": _roofline("mfma", f5, r5["event_ms_per_launch"], r5["median_ms_per_launch"])}
+    return out
 
 
 def copy_probe(torch, nbytes=256 << 20, reps=5):
@@ -209,7 +271,8 @@ def main():
                     help="also launch a 256 MiB device copy 5 times (counter calibration for profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-in-abi", action="store_true", help="skip the compile_model + container Benchmark leg")
-    ap.add_argument("--all-configs", action="store_true", help="also time the other GEMM configurations")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="time the headline configuration only (for profiler runs of one kernel)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no exchange step and every GPU box here has one "
@@ -225,24 +288,32 @@ def main():
         sys.exit(2)
     _kernels.load()
 
-    op, M, N, K, _ = SHAPES["c2a"]
+    case = GemmCase(torch, eager, _kernels, "c2a")
+    M, N, K = case.M, case.N, case.K
     if args.algo.lstrip("-").isdigit():
         algo = int(args.algo)
     else:
-        algo = _kernels.load().aitamd_gemm_find_algo(3, 0, args.algo.encode())
+        algo = _kernels.load().aitamd_gemm_find_algo(case.epi, 0, args.algo.encode())
         if algo < 0:
             sys.exit(f"bench.py: no kernel instance named {args.algo}")
     algo_given = algo >= 0
     if algo < 0 and args.select == "profile":
-        algo = pick_instance(torch, eager, _kernels, "c2a")
+        algo = case.pick_instance()
     if algo < 0:
-        algo = _kernels.load().aitamd_gemm_heuristic_algo(3, 0, 1, M, N, K, K, K, 16)
+        algo = _kernels.load().aitamd_gemm_heuristic_algo(case.epi, 0, 1, M, N, K, K, K, 16)
     if args.copy_probe:
         copy_probe(torch)
-    r = time_gemm(torch, eager, "c2a", args.steps, args.warmup, algo)
-    tflops = r["flops"] / (r["wall_ms_per_step"] * 1e-3) / 1e12
-    achieved = r["flops"] / (r["event_ms_per_launch"] * 1e-3) / 1e12
-    instance = _kernels.gemm_algo_names(3, 0)[algo]
+    r = timed_region(torch, case.step_fn(algo), args.steps, args.warmup)
+    tflops = case.flops / (r["wall_ms_per_step"] * 1e-3) / 1e12
+    instance = case.instance_name(algo)
+    roofline = _roofline("mfma", case.flops, r["event_ms_per_launch"], r["median_ms_per_launch"])
+    roofline["avg_launch_ms"] = round(r["event_ms_per_launch"], 5)
+    roofline["median_launch_ms"] = round(r["median_ms_per_launch"], 5)
+    roofline["median_of"] = f"{r['groups']} groups of consecutive launches inside the timed region"
+    traffic = MEASURED_TRAFFIC.get(instance)
+    roofline["traffic"] = traffic[0] if traffic else None
+    roofline["traffic_source"] = (f"{traffic[1]} (instance {instance})" if traffic else
+                                  f"no counter run of instance {instance} is held under profiles/")
     line = {
         "metric": "TFLOP/s + % fp16 MFMA peak, gemm_rcr_bias_gelu M=24576 K=768 N=3072",
         "value": round(tflops, 2),
@@ -261,18 +332,11 @@ def main():
                                "fp32 accumulate, tanh-GELU fused, inputs resident in HBM, rotating operand sets",
                    "instance": instance, "instance_index": algo,
                    "instance_selected_by": "--algo" if algo_given else args.select},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(instance)},
+        "roofline": roofline,
     }
-    if args.all_configs:
-        others = {}
-        for name in ("c1", "c2b", "c3"):
-            o = time_gemm(torch, eager, name, max(20, args.steps // 4), max(5, args.warmup // 4))
-            t = o["event_ms_per_launch"] * 1e-3
-            others[name] = {"op": SHAPES[name][0], "ms": round(o["event_ms_per_launch"], 5),
-                            "tflops": round(o["flops"] / t / 1e12, 2), "gbs": round(o["bytes"] / t / 1e9, 1)}
-        others.update(time_c4_c5(torch, eager, max(20, args.steps // 4), max(5, args.warmup // 4)))
-        line["other_configs"] = others
+    del case
+    if not args.no_other_configs:
+        line["other_configs"] = other_configs(torch, eager, _kernels, max(20, args.steps // 2), max(5, args.warmup // 2))
     if not args.no_in_abi:
         line["in_abi"] = in_abi(torch)
     if not args.no_cpu_baseline:

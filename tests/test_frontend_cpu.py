@@ -207,8 +207,9 @@ def test_profiler_command_line_and_instance_filter(tmp_path, monkeypatch):
         res = op.gen_profiler(str(tmp_path), DynamicProfileStrategy.MAX)
         assert len(res) == 1 and os.access(res[0][1], os.X_OK)
         assert res[0][1] == os.path.join(str(tmp_path), "profiler", "gemm_rcr_bias", op._get_profiler_filename())
-        # K = 4 leaves only the narrow-load instances
-        assert op._attrs["op_instance"] and all("_v8" not in n and "dma" not in n for n in op._attrs["op_instance"])
+        # K = 4 leaves only the instances that load narrower than 16-byte pieces along K
+        assert op._attrs["op_instance"] and all("_v8" not in n and ("dma" not in n or n.endswith("_k2"))
+                                                for n in op._attrs["op_instance"])
         cmd = op._gen_profile_cmd(os.path.dirname(res[0][1]), op._get_profiler_filename(),
                                   "M == 4096 && N == 4 && K == 4")
         assert cmd[1:] == ["gemm", "gemm_rcr_bias", "0", "4096", "4", "4"]

@@ -65,6 +65,50 @@ def test_every_instance_with_tails(algo, name, shape):
 
 
 # shapes of the reference's ROCm tests for this family
+def _k2_cases():
+    return [(i, n) for i, n in enumerate(_kernels.gemm_algo_names(1, 0)) if n.endswith("_k2")]
+
+
+@pytest.mark.parametrize("algo,name", _k2_cases())
+@pytest.mark.parametrize("shape", [(300, 264, 202), (64, 522, 1028), (515, 41, 70), (130, 200, 6), (257, 130, 8314)])
+def test_dword_aligned_k_instances(algo, name, shape):
+    """K % 8 in {2, 4, 6}: rows of A and B start 4, 8 or 12 bytes off a 16-byte boundary.  The direct-to-LDS
+    instances for such K load whole 16-byte pieces at dword-aligned addresses and take the 2, 4 or 6 elements
+    behind them with dword loads; an Inf at the start of one row must stay in that row's results (the elements
+    that follow a row's end in memory are the next row's first ones)."""
+    M, N, K = shape
+    print(f"case instance={name} M={M} N={N} K={K}", flush=True)
+    lib = _kernels.load()
+    assert lib.aitamd_gemm_algo_supported(1, 0, algo, M, N, K, K, K, 4)
+    assert not lib.aitamd_gemm_algo_supported(1, 0, algo, M, N, K + 1, K + 1, K + 1, 4)   # odd K: 2-byte rows
+    x = _rand((M, K), torch.float16, algo)
+    w = _rand((N, K), torch.float16, algo + 1, scale=K ** -0.5)
+    b = _rand((N,), torch.float16, algo + 2)
+    hot = min(5, M - 1)
+    x[hot, :min(6, K)] = float("inf")
+    want = oracle.torch_gemm("gemm_rcr_bias", x, w, b).half().float()
+    got = eager.gemm("gemm_rcr_bias", x.cuda(), w.cuda(), b.cuda(), algo=algo).cpu().float()
+    keep = [r for r in range(M) if r != hot]
+    torch.testing.assert_close(got[keep], want[keep], atol=ATOL, rtol=RTOL)
+    assert not torch.isfinite(got[hot]).any()
+
+
+@pytest.mark.parametrize("N,K", [(8314, 3072), (6912, 8314)])
+@pytest.mark.parametrize("M", [1, 2048])
+def test_reference_gemm_benchmark_shapes(M, N, K):
+    """The reference's own GEMM benchmark (tests/unittest/benchmark/test_gemm_benchmark.py:31-37): gemm_rcr with
+    N = 8314 (rows of the output start off 16-byte boundaries) and K = 8314 (so do the rows of both operands), on
+    the instance the library picks.  |x.w| sums 8314 products: the tolerance is relative to sqrt(K) rounding."""
+    print(f"case reference benchmark gemm_rcr M={M} N={N} K={K}", flush=True)
+    lib = _kernels.load()
+    algo = lib.aitamd_gemm_heuristic_algo(0, 0, 1, M, N, K, K, K, 4 if K % 8 else 16)
+    name = _kernels.gemm_algo_names(0, 0)[algo]
+    print(f"  instance {name}", flush=True)
+    if K % 8:
+        assert name.endswith("_k2"), name
+    _run_and_check("gemm_rcr", M, N, K, seed=7)
+
+
 @pytest.mark.parametrize("op,M,N,K", [
     ("gemm_rcr", 1024, 512, 256),            # test_gemm.py:83-84
     ("gemm_rcr_bias", 4096, 4, 4),           # test_gemm_bias.py:96-99
