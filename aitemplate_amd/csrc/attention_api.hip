@@ -37,7 +37,7 @@ struct TileOf {
 };
 constexpr int wide_bn(int ks, int ot) { return (16 * ks + 32 * ot) <= 128 ? 128 : 64; }
 constexpr bool wide_fits(int ks, int ot) {  // four stages of the wide tile within the LDS
-  return 4 * wide_bn(ks, ot) * (16 * ks + 8 + 32 * ot + 8) * 2 <= 160 * 1024;
+  return 4 * wide_bn(ks, ot) * (16 * ks + 8 + 32 * ot) * 2 <= 160 * 1024;
 }
 template <int KS, int OT, bool FITS = wide_fits(KS, OT)>
 struct WideTile {  // head dims too large for the wide forms keep the four-wave tile

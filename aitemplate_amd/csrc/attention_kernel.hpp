@@ -65,7 +65,15 @@ struct AttnTile {
   static constexpr int BN = BN_;          // keys per LDS tile: 128 while two workgroups still fit one CU's LDS
   static constexpr int NT = 64 * NW * NG;
   static constexpr int K_PITCH = KP + 8;  // halves; keeps 16 consecutive rows on distinct banks
-  static constexpr int V_PITCH = OP + 8;
+  // V rows carry no pad.  The transposing read fetches, per 32 lanes, 64 bytes of each of 4 consecutive rows; the
+  // four pieces have to fall into four different quarters of the 64 banks.  Rows of 64 or 192 bytes do that as
+  // they lie; rows of 128 or 256 bytes get the 64-byte pieces of a row exchanged by a row-dependent XOR.
+  static constexpr int V_PITCH = OP;
+  static constexpr int V_CR = OP / 8;                                             // 16-byte chunks per V row
+  static constexpr int V_SWZ_GROUPS = (V_CR == 8 || V_CR == 16) ? V_CR / 4 : 1;  // 64-byte pieces exchanged
+  static constexpr int V_SWZ_ROWS = V_CR == 8 ? 2 : 1;                            // rows per 256 bytes
+  // chunk index -> chunk index ^ v_swz(row)
+  static constexpr int v_swz(int row) { return 4 * ((row / V_SWZ_ROWS) % V_SWZ_GROUPS); }
   static constexpr int K_CHUNKS = BN * KP / 8;  // 16-byte chunks per tile (pads included)
   static constexpr int V_CHUNKS = BN * OP / 8;
   static constexpr int K_IT = (K_CHUNKS + NT - 1) / NT;
@@ -281,16 +289,16 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
       for (int i = 0; i < Tile::V_IT; ++i) {
         const int c = tid + i * Tile::NT;
         const int row = c / (OP / 8), col = (c % (OP / 8)) * 8;
-        if (c < Tile::V_CHUNKS) *reinterpret_cast<u32x4*>(dV + row * VPI + col) = vreg[i];
+        if (c < Tile::V_CHUNKS) *reinterpret_cast<u32x4*>(dV + row * VPI + (col ^ (Tile::v_swz(row) * 8))) = vreg[i];
       }
     };
 
     // ---- direct-to-LDS tile loader: the KL + VL wave-loads of a tile are dealt round-robin to the waves
-    constexpr int KC1 = KP / 8 + 1, VC1 = OP / 8 + 1;        // chunks per LDS row, pad chunk included
+    constexpr int KC1 = KP / 8 + 1, VC1 = OP / 8;            // chunks per LDS row (K: pad chunk included)
     constexpr int KL = BN * KC1 / 64, VL = BN * VC1 / 64;     // wave-loads per K / V tile
     constexpr int L_W = (KL + VL + NWT - 1) / NWT;
     static_assert((BN * KC1) % 64 == 0 && (BN * VC1) % 64 == 0, "tiles must be whole wave-loads");
-    static_assert(Tile::K_PITCH == KC1 * 8 && Tile::V_PITCH == VC1 * 8, "LDS rows are the chunks of a row plus one");
+    static_assert(Tile::K_PITCH == KC1 * 8 && Tile::V_PITCH == VC1 * 8, "LDS rows are whole chunks");
     typedef __attribute__((address_space(3))) void lds_void;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int wave_ld = __builtin_amdgcn_readfirstlane(wave_all);  // the loads are dealt over all waves
@@ -303,7 +311,9 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         const int idx = (is_k ? j : j - KL) * 64 + lane;
         const int c1 = is_k ? KC1 : VC1;
         const int dim = is_k ? p.K : p.O;
-        const int row = idx / c1, c = idx - row * c1;
+        const int row = idx / c1;
+        // the lane fills chunk slot idx - row * c1 of the row; for V that slot holds chunk slot ^ v_swz(row)
+        const int c = is_k ? idx - row * c1 : (idx - row * c1) ^ Tile::v_swz(row);
         d_off[i] = (c * 8 < dim) ? (uint32_t)((row * dim + c * 8) * 2) : kOobOffset;
       }
     }
@@ -371,6 +381,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     const int tr_i = lane & 15;
     const int tr_row = tr_i >> 2;
     const int tr_col = ((lane >> 4) & 1) * 16 + (tr_i & 3) * 4;
+    // every row a lane reads is its tr_row plus a multiple of 4: one swizzle value per lane
+    const int tr_swz = Tile::v_swz(tr_row) * 8;
 
     // 32-key sub-blocks per softmax step: two for head dims up to 48, which halves the per-step work (exchange
     // across halves, rescale test, branches) per key: 3.7 % faster at head dim 40; at 64 the 16 extra
@@ -494,7 +506,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         for (int st = 0; st < 2 * KB; ++st) {
 #pragma unroll
           for (int ot = 0; ot < OT; ++ot) {
-            const T* vb = cV + (blk * KB * 32 + st * 16 + h * 4 + tr_row) * VPI + ot * 32 + tr_col;
+            const T* vb = cV + (blk * KB * 32 + st * 16 + h * 4 + tr_row) * VPI + ((ot * 32) ^ tr_swz) + tr_col;
             const vec4 lo = AttnVec<T>::tr_read(vb);
             const vec4 hi = AttnVec<T>::tr_read(vb + 8 * VPI);
             vec8 vf;

@@ -200,3 +200,25 @@ def test_config_c5_full_size():
     torch.cuda.synchronize()
     assert got.shape == (2, 4096, 8, 40)
     torch.testing.assert_close(got.cpu().float(), want, atol=TOL, rtol=TOL)
+
+
+def test_nan_in_a_key_gives_nan_for_its_batch_entry_only():
+    """A NaN score stays a NaN here, as in PyTorch's softmax (the oracle): every query of the batch entry that
+    holds the bad key row comes out NaN, the other batch entries are untouched.  Composable Kernel, which the
+    reference calls, resets NaN scores to -inf before the softmax instead
+    (python/aitemplate/utils/mk_ck_lib/gemm_operation.py:415-424 instantiates that kernel); that reset is not
+    replicated, and this test pins the difference."""
+    B, M, N, K, O, G = 4, 96, 200, 64, 64, 2
+    print(f"case attention NaN key B={B} M={M} N={N} K={K}", flush=True)
+    q, k, v = _rand((B, M, K), torch.float16, 11), _rand((B, N, K), torch.float16, 12), _rand((B, N, O), torch.float16, 13)
+    k[1, 77, 5] = float("nan")
+    want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, K ** -0.5, G, False).half().float()   # [B/G, M, G, O]
+    got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
+    assert torch.isnan(want[0, :, 1, :]).all(), "the oracle (PyTorch softmax) propagates the NaN"
+    assert torch.isnan(got[0, :, 1, :]).all()
+    keep = torch.ones(B // G, G, dtype=torch.bool)
+    keep[0, 1] = False
+    for bo in range(B // G):
+        for g in range(G):
+            if keep[bo, g]:
+                torch.testing.assert_close(got[bo, :, g, :], want[bo, :, g, :], atol=TOL, rtol=TOL)

@@ -69,6 +69,57 @@ def _run_gemm_case(op_name, Ms, N, K, dtype="float16", tol=1e-2):
     module.close()
 
 
+def test_second_compile_of_the_same_graph_runs_no_profiler(tmp_path, monkeypatch):
+    """The profiling-result cache across compile_model calls (reference flow: gemm_common.py:618-676 with the
+    database of backend/profiler_cache.py): the first build times every instance of its two ops, the second build
+    of the same graph finds both workloads in the database, starts no profiler and picks the same instances, so
+    the two model libraries give bit-identical results."""
+    from aitemplate_amd.backend.profiler_runner import ProfilerRunner
+
+    monkeypatch.delenv("CI_FLAG", raising=False)
+    monkeypatch.delenv("FORCE_PROFILE", raising=False)
+    monkeypatch.setenv("CACHE_DIR", str(tmp_path / "cache"))
+    pushes = []
+    real_push = ProfilerRunner.push
+
+    def counting_push(self, cmds, *args, **kwargs):
+        pushes.append(list(cmds))
+        return real_push(self, cmds, *args, **kwargs)
+
+    monkeypatch.setattr(ProfilerRunner, "push", counting_push)
+    M, K, H, N = 384, 256, 512, 128
+
+    def build(tag):
+        X = Tensor([M, K], name="x", is_input=True)
+        W0, B0 = Tensor([H, K], name="w0", is_input=True), Tensor([H], name="b0", is_input=True)
+        W1, B1 = Tensor([N, H], name="w1", is_input=True), Tensor([N], name="b1", is_input=True)
+        Y = _mark_output(ops.gemm_rcr_bias()(ops.gemm_rcr_bias_fast_gelu()(X, W0, B0), W1, B1), "y")
+        module = compile_model(Y, detect_target(), str(tmp_path), f"cache_{tag}")
+        picked = [op._attrs["exec_path"][k].algo for op in [list(Y.src_ops())[0]] for k in op._attrs["exec_path"]]
+        return module, picked
+
+    x, w0, b0 = _rand((M, K), 1), _rand((H, K), 2, K ** -0.5), _rand((H,), 3)
+    w1, b1 = _rand((N, H), 4, H ** -0.5), _rand((N,), 5)
+    ins = {"x": x.cuda(), "w0": w0.cuda(), "b0": b0.cuda(), "w1": w1.cuda(), "b1": b1.cuda()}
+    outs = []
+    first, picked_first = build("first")
+    n_first = len(pushes)
+    assert n_first >= 2, "the first build profiles both ops"
+    assert os.path.isfile(tmp_path / "cache" / "rocm.db")
+    second, picked_second = build("second")
+    assert len(pushes) == n_first, f"the second build started profilers: {pushes[n_first:]}"
+    assert picked_second == picked_first
+    for module in (first, second):
+        y = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        module.run_with_tensors(ins, [y])
+        outs.append(y.cpu())
+        module.close()
+    assert torch.equal(outs[0], outs[1])
+    h = oracle.torch_gemm("gemm_rcr_bias_fast_gelu", x, w0, b0).half()
+    want = oracle.torch_gemm("gemm_rcr_bias", h, w1, b1).half().float()
+    torch.testing.assert_close(outs[0].float(), want, atol=1e-2, rtol=1e-2)
+
+
 def test_split_k_instance_through_compile_model():
     """A few tiles with a very long K: the profiler finds a split-K instance fastest, its WS:<bytes> becomes the
     op's `workspace` attribute, the model allocates that once and hands it to the op function (the reference's
