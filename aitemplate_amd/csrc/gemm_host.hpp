@@ -30,6 +30,18 @@ struct GemmAlgoTable {
   int count;
 };
 
+// Workgroups per tile of a split-K launch (the launcher and the instance choice share the rule): as many as bring
+// the grid up to about one workgroup per CU, each with at least two K-slabs, at most 16; 1 (no splitting, nothing
+// written to the scratch memory) for grids that fill the device anyway.  Measured against two and four workgroups
+// per CU and against longer minimum shares (256x1024x1024, 512x768x3072, 1x6912x8314, 64x256x8192): never slower.
+inline int split_k_rule(int64_t tiles, int64_t k_tiles, int cus) {
+  if (tiles <= 0) return 1;
+  int64_t s = cus / tiles;
+  if (s > k_tiles / 2) s = k_tiles / 2;
+  if (s > 16) s = 16;
+  return (int)(s < 1 ? 1 : s);
+}
+
 // Defined once per (epilogue, dtype) translation unit; nullptr table when that
 // combination is not compiled in.
 GemmAlgoTable gemm_table(int epilogue, int dtype);

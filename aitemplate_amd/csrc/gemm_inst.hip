@@ -76,9 +76,9 @@ template <class Tile>
 struct IsSplitK {
   static constexpr bool value = false;
 };
-template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX>
-struct IsSplitK<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, 1>> {
-  static constexpr bool value = true;
+template <int BM, int BN, int BK, int WM, int WN, int NS, int OCC, int PIPE, int MT, int AUX, int MODE>
+struct IsSplitK<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>> {
+  static constexpr bool value = (MODE & 1) != 0;
 };
 template <class Tile>
 struct IsPersistent {
@@ -106,12 +106,8 @@ inline int device_cus(int dev) {
 template <class Tile>
 int split_k_factor(const GemmParams& p, int cus) {
   const int64_t tiles = (int64_t)((p.M + Tile::BM - 1) / Tile::BM) * ((p.N + Tile::BN - 1) / Tile::BN) * p.batch;
-  const int64_t k_tiles = (p.K + Tile::BK - 1) / Tile::BK;
-  if (tiles <= 0) return 1;
-  int64_t s = cus / tiles;
-  if (s > k_tiles / 2) s = k_tiles / 2;
-  if (s > 16) s = 16;
-  return (int)(s < 1 ? 1 : s);
+  const int64_t k_tiles = ((Tile::KVEC == 8 ? p.K : (p.K & ~7)) + Tile::BK - 1) / Tile::BK;
+  return split_k_rule(tiles, k_tiles, cus);
 }
 template <class Tile>
 int64_t workspace_of(const GemmParams& p) {
@@ -255,10 +251,20 @@ const GemmAlgo kAlgos[] = {
    dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>::NT, OCC,                        \
                   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>::kLdsBytes),                      \
    1, 1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 2>>, nullptr},
+#define AITAMD_GEMM_TILE_DMA_SPLITK_K2(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT)                                \
+  {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
+   "_k2_splitk",                                                                                          \
+   BM, BN, BK, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 3>::NT, 2,                             \
+   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 3>::kLdsBytes,                                     \
+   dma_wgs_per_cu(GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 3>::NT, OCC,                        \
+                  GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 3>::kLdsBytes),                      \
+   4, 1, &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 3>>,                             \
+   &workspace_of<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, 0, 3>>},
 #include "gemm_tiles.inc"
 #undef AITAMD_GEMM_TILE
 #undef AITAMD_GEMM_TILE_DMA
 #undef AITAMD_GEMM_TILE_DMA_K2
+#undef AITAMD_GEMM_TILE_DMA_SPLITK_K2
 #undef AITAMD_GEMM_TILE_PERSIST
 #undef AITAMD_GEMM_TILE_DMA_SPLITK
 };

@@ -26,7 +26,7 @@ namespace aitamd {
 // included, so the result does not depend on who came last) and runs the epilogue.  Nobody waits for anybody.
 // For grids that leave most CUs idle and tiles small enough that a partial tile is a few KiB.
 //
-// MODE 2, K in dwords: K, the row pitches and the operand pointers need to be whole dwords only (K % 8 in {2, 4, 6}:
+// MODE 2, K in dwords (3: both): K, the row pitches and the operand pointers need to be whole dwords only (K % 8 in {2, 4, 6}:
 // rows that start 4, 8 or 12 bytes off a 16-byte boundary).  The 16-byte slab loads take dword-aligned addresses
 // as they are; the K loop runs over the whole 16-byte pieces of a row, and the 2, 4 or 6 elements behind them are
 // fetched once per tile with dword loads straight into MFMA operands (lanes of the first k-chunk, zeros elsewhere)
@@ -34,8 +34,8 @@ namespace aitamd {
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int OCC_, int PIPE_ = 0, int MT_ = 32, int AUX_ = 0,
           int MODE_ = 0>
 struct GemmTileDma {
-  static constexpr int SPLITK = MODE_ == 1;
-  static constexpr int KTAIL = MODE_ == 2;
+  static constexpr int SPLITK = MODE_ & 1;          // MODE bit 0
+  static constexpr int KTAIL = (MODE_ >> 1) & 1;    // MODE bit 1
   static constexpr int64_t kSlotBytes = (int64_t)BM_ * BN_ * 4;
   static constexpr int64_t kCounterAlign = 4096;
   // scratch bytes for `tiles` (batch x tile) pairs shared by `splits` workgroups each: one counter per pair,
@@ -439,7 +439,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     if constexpr (Tile::KTAIL != 0) {
-      if (k_main < p.K) {
+      // (of the workgroups that share a tile's K range the last one takes the tail)
+      if (k_main < p.K && (Tile::SPLITK == 0 || split == splits - 1)) {
         vec8 ta[MI], tb[NI];
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)

@@ -53,6 +53,30 @@ def test_splitk_matches_oracle(op, nres, M, N, K):
         assert int(scratch[:counter_bytes].to(torch.int32).sum()) == 0
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 6912, 8314), (100, 200, 4102), (64, 64, 270), (48, 136, 12)])
+def test_splitk_with_dword_aligned_k(M, N, K):
+    """K % 8 in {2, 4, 6}: only the instance that takes rows aligned to dwords qualifies; the workgroup with the
+    last share of K multiplies the 2, 4 or 6 elements behind the rows' last whole 16-byte piece."""
+    op = "gemm_rcr_bias"
+    algos = [(i, n) for i, n in _splitk_algos(op) if n.endswith("_k2_splitk")]
+    assert algos, "no split-K instance for dword-aligned K compiled"
+    lib = _kernels.load()
+    x, w, b, _ = _inputs(M, N, K, 0, torch.float16, seed=M + N + K)
+    want = oracle.torch_gemm(op, x, w, b).half().float()
+    xs, ws, bs = x.cuda(), w.cuda(), b.cuda()
+    for algo, name in algos:
+        assert lib.aitamd_gemm_algo_supported(_kernels.EPILOGUE_OF_OP[op], 0, algo, M, N, K, K, K, 4)
+        need = eager.gemm_workspace_bytes(op, algo, M, N, K)
+        scratch = eager.new_workspace(need)
+        print(f"case {op} {name} M={M} N={N} K={K} workspace={need}", flush=True)
+        for rep in range(2):
+            out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+            eager.gemm(op, xs, ws, bs, out=out, algo=algo, workspace=scratch)
+            torch.cuda.synchronize()
+            torch.testing.assert_close(out.cpu().float(), want, atol=1e-2, rtol=1e-2)
+        assert int(scratch[:min(need, 4096)].to(torch.int32).sum()) == 0
+
+
 def test_splitk_is_deterministic_and_bf16():
     op, (M, N, K) = "gemm_rcr_bias", (192, 320, 2048)
     x, w, b, _ = _inputs(M, N, K, 0, torch.bfloat16, seed=5)
