@@ -132,13 +132,19 @@ class GemmCase:
                  workspace=ws)
         return step
 
+    @property
+    def launch_bound(self):
+        """A launch lasts a few microseconds: only a replayed graph lets the GPU, not the host, set the pace."""
+        return self.flops < 5e9
+
     def pick_instance(self, iters=15):
         """Untimed selection pass, the same procedure compile_model's profiling step applies
         (python/aitemplate/compiler/ops/gemm_universal/gemm_common.py:743-829 in the reference):
         time every instance that supports the problem and keep the fastest."""
         best, best_ms = -1, float("inf")
         for algo in self.supported:
-            ms = timed_region(self.torch, self.step_fn(algo), iters, 3, groups=1)["event_ms_per_launch"]
+            ms = timed_region(self.torch, self.step_fn(algo), iters * (4 if self.launch_bound else 1), 3, groups=1,
+                              graph=self.launch_bound)["event_ms_per_launch"]
             if ms < best_ms:
                 best, best_ms = algo, ms
         return best
@@ -161,8 +167,7 @@ def other_configs(torch, eager, kernels, steps, warmup):
     for name in ("c1", "c2b", "c3"):
         case = GemmCase(torch, eager, kernels, name)
         algo = case.pick_instance()
-        # a launch of config 1 lasts a few microseconds: replay a captured graph so the GPU, not the host, sets the pace
-        graph = name == "c1"
+        graph = case.launch_bound  # (config 1)
         r = timed_region(torch, case.step_fn(algo), steps, warmup, graph=graph)
         ws = eager.gemm_workspace_bytes(case.op, algo, case.M, case.N, case.K)
         out[name] = {"op": case.op, "M": case.M, "N": case.N, "K": case.K, "instance": case.instance_name(algo),
