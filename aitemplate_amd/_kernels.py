@@ -85,6 +85,8 @@ EXPORTED_SYMBOLS = [
     "aitamd_bmm_softmax_bmm_permute",
     "aitamd_mem_eff_attention",
     "aitamd_attention_set_variant",
+    "aitamd_elementwise",
+    "aitamd_elementwise_supported",
     "aitamd_gemm_workspace_bytes",
     "aitamd_gemm_rcr_ws",
     "aitamd_gemm_rcr_noalloc",
@@ -160,6 +162,10 @@ def load() -> ctypes.CDLL:
         lib.aitamd_gemm_noalloc_scratch_bytes.argtypes = []
         lib.aitamd_attention_set_variant.restype = i32
         lib.aitamd_attention_set_variant.argtypes = [i32]
+        lib.aitamd_elementwise.restype = i32
+        lib.aitamd_elementwise.argtypes = [i32, i32, vp, vp, vp, i64, i64, ctypes.c_float, i32, vp]
+        lib.aitamd_elementwise_supported.restype = i32
+        lib.aitamd_elementwise_supported.argtypes = [i32]
         _lib = lib
         return lib
 

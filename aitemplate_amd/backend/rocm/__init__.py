@@ -1,2 +1,2 @@
-from . import attention, gemm  # noqa: F401  (registers the rocm.* hooks)
+from . import attention, elementwise, gemm  # noqa: F401  (registers the rocm.* hooks)
 from .target_def import ROCM  # noqa: F401

@@ -75,7 +75,7 @@ def compile_model(
             _bind_constants(graph, constants)
             if do_optimize_graph:
                 graph = transform.fuse_mm_elementwise(graph, output_tensors)
-            transform.check_no_elementwise_left(graph)
+            transform.check_leftover_elementwise(graph)
             # last-dim split / concatenate become offsets and row pitches of the GEMM ops around them
             graph = transform.fuse_strided_views(graph, output_tensors)
             transform.name_graph(graph)

@@ -5,5 +5,5 @@ from .refine_graph import refine_graph  # noqa: F401
 from .toposort import toposort  # noqa: F401
 from .mark_param_tensor import mark_param_tensor  # noqa: F401
 from .transform_utils import get_sorted_ops  # noqa: F401
-from .fuse_mm_elementwise import check_no_elementwise_left, fuse_mm_elementwise  # noqa: F401
+from .fuse_mm_elementwise import check_leftover_elementwise, fuse_mm_elementwise  # noqa: F401
 from .fuse_strided_views import fuse_strided_views  # noqa: F401

@@ -158,11 +158,15 @@ def fuse_mm_elementwise(sorted_graph: List[Tensor], output_tensors: List[Tensor]
     return sorted_graph
 
 
-def check_no_elementwise_left(sorted_graph: List[Tensor]) -> None:
+def check_leftover_elementwise(sorted_graph: List[Tensor]) -> None:
+    """Element-wise ops that no epilogue absorbed run as stand-alone launches; raise for those the stand-alone
+    kernel cannot take, naming the tensor."""
     for t in sorted_graph:
         for op in t.src_ops():
             if op._attrs["op"] == "elementwise":
-                raise NotImplementedError(
-                    f"elementwise({op._attrs['func'].name}) producing {t._attrs['name'] or 'an unnamed tensor'} "
-                    "could not be fused into a GEMM epilogue, and this backend has no stand-alone element-wise "
-                    "kernels")
+                try:
+                    op.standalone_plan()
+                except NotImplementedError as e:
+                    raise NotImplementedError(
+                        f"{e}; the op producing {t._attrs['name'] or 'an unnamed tensor'} could not be fused into a "
+                        "GEMM epilogue either") from None

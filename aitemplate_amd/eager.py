@@ -348,3 +348,41 @@ def mem_eff_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal:
                                       _p(lengths_kv), _p(lengths_q), _stream_ptr())
     _kernels.check(rc, "mem_eff_attention")
     return out
+
+
+def elementwise(func: str, a: torch.Tensor, b=None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Stand-alone element-wise op `func` (a FuncEnum name, e.g. "ADD", "FASTGELU"): f(a, b) with b a tensor whose
+    shape is a's or a suffix of it (leading 1s allowed), a number, or None for the unary functions.  A number or a
+    broadcast tensor as the FIRST operand: pass it as `a` and the full-shape tensor as `b`."""
+    from .compiler.ops.common.epilogue import FuncEnum
+
+    lib = _kernels.load()
+    fid = FuncEnum[func].value
+    swap = 0
+    if not isinstance(a, torch.Tensor) or (isinstance(b, torch.Tensor) and b.numel() > a.numel()):
+        a, b, swap = b, a, 1
+    _check(a, "a", None)
+    if a.dtype not in _TORCH_DTYPE_ID or not a.is_contiguous():
+        raise ValueError("a must be a contiguous fp16 / bf16 GPU tensor")
+    b_ptr, b_period, b_value = None, 1, 0.0
+    if isinstance(b, torch.Tensor):
+        _check(b, "b", a.dtype)
+        if not b.is_contiguous():
+            raise ValueError("b must be contiguous")
+        shape = list(b.shape)
+        while shape and shape[0] == 1:
+            shape.pop(0)
+        if shape != list(a.shape)[len(a.shape) - len(shape):]:
+            raise ValueError(f"b of shape {tuple(b.shape)} does not broadcast over the leading dims of {tuple(a.shape)}")
+        b_ptr, b_period = _p(b), max(1, b.numel())
+    elif b is not None:
+        b_value = float(b)
+    if out is None:
+        out = torch.empty_like(a)
+    else:
+        _check(out, "out", a.dtype)
+        _check_out(out, a.numel(), "a.numel()")
+    rc = lib.aitamd_elementwise(fid, _TORCH_DTYPE_ID[a.dtype], _p(a), b_ptr, _p(out), a.numel(), b_period, b_value, swap,
+                                _stream_ptr())
+    _kernels.check(rc, f"elementwise({func})")
+    return out

@@ -262,6 +262,20 @@ AITAMD_API int aitamd_mem_eff_attention(int dtype,
  * reference (CK instances are chosen by its profiler only). */
 AITAMD_API int aitamd_attention_set_variant(int variant);
 
+/* Stand-alone element-wise op: out[i] = f(a[i], b[i % b_period]) over `numel` flattened elements (f(b, a) with
+ * swap_operands).  `func` is the reference's FuncEnum value (python/aitemplate/compiler/ops/common/epilogue.py:34-70):
+ * binary ADD 1, SUB 2, MUL 3, DIV 4, MAX 13, MIN 14 (NaN if either operand is), LRELU 16 (b: negative slope), POW 22;
+ * unary TANH 5, COS 6, SIN 7, SIGN 8, ABS 9, LOGE 10, EXP 11, SQRT 12, SIGMOID 15, RELU 18, SILU 21, GELU 23 (erf form),
+ * FASTGELU 24 (tanh form), SOFTSIGN 27, FLOOR 30, LOG1P 31, RECIPROCAL 32.  Arithmetic in fp32, one rounding.  b: a tensor of b_period elements that tiles the output (same shape: b_period =
+ * numel; an operand that broadcasts over leading dims: the product of its dims; a one-element tensor: 1), or null with
+ * the constant b_value; ignored by the unary functions.  Replaces the single-op case of the kernels the reference
+ * generates in python/aitemplate/backend/common/elementwise_common.py (ROCm entry:
+ * python/aitemplate/backend/rocm/elementwise/fused_elementwise.py:27-65). */
+AITAMD_API int aitamd_elementwise(int func, int dtype, const void* a, const void* b, void* out, int64_t numel,
+                                  int64_t b_period, float b_value, int swap_operands, void* stream);
+/* 1 when aitamd_elementwise implements FuncEnum value `func` (instance filtering at compile time). */
+AITAMD_API int aitamd_elementwise_supported(int func);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

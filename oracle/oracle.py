@@ -122,6 +122,31 @@ def torch_epilogue(op: str, y: torch.Tensor, d0=None, d1=None) -> torch.Tensor:
     raise KeyError(op)
 
 
+def torch_elementwise(func: str, a, b=None) -> torch.Tensor:
+    """f(a, b) in fp32 for the reference's FuncEnum name `func`, operands broadcast numpy-style
+    (python/aitemplate/compiler/ops/common/elementwise.py:68-87; the function table is
+    python/aitemplate/backend/backend_spec.py:117-330).  MAX / MIN return NaN when either operand is NaN
+    (fmaxf_nan / fminf_nan, backend/rocm/elementwise/custom_math.h:282-310), RELU maps NaN to 0
+    (custom_math.h:117), GELU is the erf form and FASTGELU the tanh form (hgelu / h_fast_gelu of
+    backend/cuda/elementwise/custom_math.cuh)."""
+    F = torch.nn.functional
+    x = _f(a) if isinstance(a, torch.Tensor) else torch.tensor(float(a))
+    y = None if b is None else (_f(b) if isinstance(b, torch.Tensor) else torch.tensor(float(b)))
+    table = {
+        "ADD": lambda: x + y, "SUB": lambda: x - y, "MUL": lambda: x * y, "DIV": lambda: x / y,
+        "MAX": lambda: torch.maximum(x, y), "MIN": lambda: torch.minimum(x, y),
+        "TANH": lambda: torch.tanh(x), "ABS": lambda: torch.abs(x), "EXP": lambda: torch.exp(x),
+        "SQRT": lambda: torch.sqrt(x), "SIGMOID": lambda: torch.sigmoid(x),
+        "RELU": lambda: torch.where(x > 0, x, torch.zeros_like(x)), "SILU": lambda: x * torch.sigmoid(x),
+        "GELU": lambda: F.gelu(x), "FASTGELU": lambda: F.gelu(x, approximate="tanh"),
+        "COS": lambda: torch.cos(x), "SIN": lambda: torch.sin(x), "SIGN": lambda: torch.sign(x),
+        "LOGE": lambda: torch.log(x), "LOG1P": lambda: torch.log1p(x), "POW": lambda: torch.pow(x, y),
+        "LRELU": lambda: torch.where(x > 0, x, x * y), "SOFTSIGN": lambda: x / (1 + torch.abs(x)),
+        "FLOOR": lambda: torch.floor(x), "RECIPROCAL": lambda: 1.0 / x,
+    }
+    return table[func]()
+
+
 def torch_gemm(op: str, x, w, bias=None, d0=None, d1=None) -> torch.Tensor:
     """fp32 result of reference op `op`; cast to the input dtype by the caller."""
     y = torch.nn.functional.linear(_f(x), _f(w), _f(bias) if op != "gemm_rcr" else None)

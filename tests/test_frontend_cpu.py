@@ -866,7 +866,7 @@ def test_fuse_mm_elementwise_patterns(funcs, fused):
     assert op._attrs["inputs"][:3] == [X, W, Bv] and op._attrs["inputs"][3:] == residuals
     for t in (X, W, Bv, *residuals):
         assert list(t.dst_ops()) == [op]  # the replaced ops no longer hang off the inputs
-    transform.check_no_elementwise_left(graph)
+    transform.check_leftover_elementwise(graph)
 
 
 def test_fuse_mm_elementwise_bias_swish_operators_and_limits():
@@ -886,8 +886,7 @@ def test_fuse_mm_elementwise_bias_swish_operators_and_limits():
     r._attrs["is_output"] = True
     graph, outs = _fuse([h, r])
     assert _op_names(graph) == ["gemm_rcr_bias", "elementwise"]
-    with pytest.raises(NotImplementedError, match="could not be fused"):
-        transform.check_no_elementwise_left(graph)
+    transform.check_leftover_elementwise(graph)  # the left-over RELU runs as a stand-alone launch
     # a residual of another shape (row broadcast) is not an epilogue of this backend
     h2 = ops.gemm_rcr_bias()(X, W, Bv)
     z = h2 + Tensor([1, N], name="row", is_input=True)
@@ -925,7 +924,64 @@ def test_compile_model_runs_the_fusion_pass_and_rejects_leftovers(tmp_path, monk
             compile_model(y, detect_target(), str(tmp_path), "fused")
     model_src = (tmp_path / "fused" / "model-generated.cpp").read_text()
     assert re.findall(r'OpEntry\{"(\w+)"', model_src) == ["gemm_rcr_bias_relu_0"]
-    z = ops.elementwise(ops.FuncEnum.EXP)(nn.Linear(32, 48)(Tensor([64, 32], name="x2", is_input=True)))
+    # a function without a stand-alone kernel, and a broadcast the stand-alone kernel cannot tile
+    z = ops.elementwise(ops.FuncEnum.ELU)(nn.Linear(32, 48)(Tensor([64, 32], name="x2", is_input=True)))
     z._attrs["is_output"] = True
-    with pytest.raises(NotImplementedError, match="could not be fused"):
+    with pytest.raises(NotImplementedError, match="no stand-alone kernel.*could not be fused"):
         compile_model(z, detect_target(), str(tmp_path), "leftover")
+    col = Tensor([64, 1], name="col", is_input=True)
+    z = ops.elementwise(ops.FuncEnum.EXP)(nn.Linear(32, 48)(Tensor([64, 32], name="x3", is_input=True))) * col
+    z._attrs["is_output"] = True
+    with pytest.raises(NotImplementedError, match="does not tile.*could not be fused"):
+        compile_model(z, detect_target(), str(tmp_path), "leftover2")
+
+
+def test_leftover_elementwise_ops_become_standalone_launches(tmp_path, monkeypatch):
+    """Counterpart of the reference's fused_elementwise code generation
+    (backend/rocm/elementwise/fused_elementwise.py) for ops no GEMM epilogue absorbed: one launch each."""
+    from aitemplate_amd import _kernels
+    from aitemplate_amd.compiler.ops.common.elementwise import STANDALONE_FUNCS, standalone_plan
+
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    reset_name_counters()
+    lib = _kernels.load()
+    assert {f.value for f in ops.FuncEnum if lib.aitamd_elementwise_supported(f.value)} == \
+        {f.value for f in STANDALONE_FUNCS}
+    B = IntVar([1, 8], name="batch")
+    X = Tensor([B, 64, 32], name="x", is_input=True)
+    row = Tensor([1, 48], name="row", is_input=True)
+    lin = nn.Linear(32, 48)
+    lin.name_parameter_tensor("fc")
+    h = lin(X)
+    h._attrs["is_output"] = True  # two consumers: the chain cannot fold into the GEMM
+    h._attrs["name"] = "h"
+    e = ops.elementwise(ops.FuncEnum.EXP)(h)
+    s = 2.0 - e  # constant first: f(b, a)
+    r = ops.elementwise(ops.FuncEnum.MAX)(row, s)  # broadcast operand first
+    y = r / h  # same shape
+    y._attrs["is_output"] = True
+    y._attrs["name"] = "y"
+    plans = []
+    for t in (e, s, r, y):
+        a, b, value, swap = standalone_plan(list(t.src_ops())[0]._attrs)
+        plans.append((a is h or a is e or a is s or a is r, None if b is None else b._attrs["name"], value, swap))
+    assert plans == [(True, None, 0.0, 0), (True, None, 2.0, 1), (True, "row", 0.0, 1), (True, "h", 0.0, 0)]
+    import torch
+
+    if torch.cuda.is_available():
+        compile_model([h, y], detect_target(), str(tmp_path), "ew").close()
+    else:
+        with pytest.raises(RuntimeError, match="AITemplateModelContainerCreate"):
+            compile_model([h, y], detect_target(), str(tmp_path), "ew")
+    model_src = (tmp_path / "ew" / "model-generated.cpp").read_text()
+    assert re.findall(r'OpEntry\{"(\w+)"', model_src) == ["gemm_rcr_bias_0", "elementwise_1", "elementwise_2",
+                                                          "elementwise_3", "elementwise_4"]
+    assert "elementwise_3(" in model_src and "row, batch * " in model_src.replace("\n", " ")
+    src = (tmp_path / "ew" / "elementwise_2.cpp").read_text()
+    assert "aitamd_elementwise(2 /* SUB */, 0, a, b, out, numel, b_period" in src and "2.0f, 1, stream" in src
+    # both operands broadcast, and an operand that broadcasts over an inner dim, are refused with the reason
+    with pytest.raises(NotImplementedError, match="both broadcast"):
+        list((Tensor([4, 1], name="p", is_input=True) + Tensor([1, 6], name="q", is_input=True)).src_ops())[0] \
+            .standalone_plan()
+    with pytest.raises(NotImplementedError, match="with 2 operands is not supported"):
+        list(ops.elementwise(ops.FuncEnum.RELU)(h, h).src_ops())[0].standalone_plan()
