@@ -45,6 +45,9 @@ struct ElemTraits<f16> {
   }
   static AITAMD_DEVICE float to_float(f16 v) { return (float)v; }
   static AITAMD_DEVICE f16 from_float(float v) { return (f16)v; }
+  // float(v) + c in one instruction: with `one` = 1.0 in a register the compiler cannot see through, the fused
+  // multiply-add of a widened half maps to v_fma_mix_f32 (conversion and add together; same single rounding)
+  static AITAMD_DEVICE float to_float_plus(f16 v, float one, float c) { return __builtin_fmaf((float)v, one, c); }
 };
 
 template <>
@@ -59,6 +62,7 @@ struct ElemTraits<bf16> {
   }
   static AITAMD_DEVICE float to_float(bf16 v) { return (float)v; }
   static AITAMD_DEVICE bf16 from_float(float v) { return (bf16)v; }
+  static AITAMD_DEVICE float to_float_plus(bf16 v, float one, float c) { (void)one; return (float)v + c; }
 };
 
 // LDS transpose read: 4 x 16-bit per lane, gathered across the 16 lanes of a block
@@ -89,8 +93,17 @@ AITAMD_DEVICE typename ElemTraits<T>::vec8 join_halves(typename ElemTraits<T>::v
 // ---------------------------------------------------------------------------
 constexpr uint32_t kOobOffset = 0x80000000u;  // >= any num_records we build
 
+// Every descriptor in these kernels is the same for all lanes of a wave (one per tile, batch entry or wave
+// part), but the compiler cannot prove that for values computed from the wave index or loaded tile coordinates,
+// and a buffer access through a descriptor it takes for lane-varying is wrapped in a loop over the wave's
+// distinct descriptors (four v_readfirstlane, two 64-bit compares and a branch per access).  Reading base and
+// size from the first lane states the uniformity; where they already are scalar registers this folds away.
 AITAMD_DEVICE __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t num_bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, num_bytes, 0x00020000);
+  const uint64_t v = reinterpret_cast<uint64_t>(base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uint64_t)hi << 32) | lo), 0,
+                                           __builtin_amdgcn_readfirstlane(num_bytes), 0x00020000);
 }
 
 AITAMD_DEVICE u32x4 buffer_load_16B(__amdgpu_buffer_rsrc_t r, uint32_t voffset) {

@@ -69,37 +69,53 @@ AITAMD_DEVICE float hardswish_f(float x) {
 template <int kId>
 struct Epilogue;
 
-#define AITAMD_DEF_EPI(ID, BIAS, ND, EXPR)                                         \
+// LEAD: how many of the residuals the expression adds, in order, right behind acc (+ b).  A caller may fold those
+// adds into its conversion of the residuals (v_fma_mix: half -> float and add in one instruction, the same single
+// rounding) and pass -0.0, which adds nothing, in their place.
+#define AITAMD_DEF_EPI(ID, BIAS, ND, LEAD, EXPR)                                   \
   template <>                                                                  \
   struct Epilogue<ID> {                                                        \
     static constexpr int kId = ID;                                             \
     static constexpr bool kHasBias = BIAS;                                     \
     static constexpr int kNumD = ND;                                           \
+    static constexpr int kLeadingAdds = LEAD;                                  \
     static AITAMD_DEVICE float apply(float acc, float b, float d0, float d1) { \
       (void)b; (void)d0; (void)d1;                                             \
       return EXPR;                                                             \
     }                                                                          \
   };
 
-AITAMD_DEF_EPI(kEpiNone, false, 0, acc)
-AITAMD_DEF_EPI(kEpiBias, true, 0, acc + b)
-AITAMD_DEF_EPI(kEpiBiasRelu, true, 0, fmaxf(acc + b, 0.0f))
-AITAMD_DEF_EPI(kEpiBiasGelu, true, 0, gelu_tanh(acc + b))
-AITAMD_DEF_EPI(kEpiBiasAdd, true, 1, (acc + b) + d0)
-AITAMD_DEF_EPI(kEpiBiasAddAdd, true, 2, ((acc + b) + d0) + d1)
-AITAMD_DEF_EPI(kEpiBiasAddRelu, true, 1, fmaxf((acc + b) + d0, 0.0f))
-AITAMD_DEF_EPI(kEpiBiasAddAddRelu, true, 2, fmaxf(((acc + b) + d0) + d1, 0.0f))
-AITAMD_DEF_EPI(kEpiBiasSigmoid, true, 0, sigmoid_f(acc + b))
-AITAMD_DEF_EPI(kEpiBiasTanh, true, 0, tanh_f(acc + b))
-AITAMD_DEF_EPI(kEpiBiasSwish, true, 0, (acc + b) * sigmoid_f(acc + b))
-AITAMD_DEF_EPI(kEpiBiasHardswish, true, 0, hardswish_f(acc + b))
-AITAMD_DEF_EPI(kEpiBiasMul, true, 1, (acc + b) * d0)
-AITAMD_DEF_EPI(kEpiBiasMulAdd, true, 2, (acc + b) * d0 + d1)
-AITAMD_DEF_EPI(kEpiBiasSigmoidMul, true, 1, sigmoid_f(acc + b) * d0)
-AITAMD_DEF_EPI(kEpiBiasSigmoidMulTanh, true, 1, tanh_f(sigmoid_f(acc + b) * d0))
-AITAMD_DEF_EPI(kEpiBiasMulTanh, true, 1, tanh_f((acc + b) * d0))
-AITAMD_DEF_EPI(kEpiAdd, false, 1, acc + d0)
+AITAMD_DEF_EPI(kEpiNone, false, 0, 0, acc)
+AITAMD_DEF_EPI(kEpiBias, true, 0, 0, acc + b)
+AITAMD_DEF_EPI(kEpiBiasRelu, true, 0, 0, fmaxf(acc + b, 0.0f))
+AITAMD_DEF_EPI(kEpiBiasGelu, true, 0, 0, gelu_tanh(acc + b))
+AITAMD_DEF_EPI(kEpiBiasAdd, true, 1, 1, (acc + b) + d0)
+AITAMD_DEF_EPI(kEpiBiasAddAdd, true, 2, 2, ((acc + b) + d0) + d1)
+AITAMD_DEF_EPI(kEpiBiasAddRelu, true, 1, 1, fmaxf((acc + b) + d0, 0.0f))
+AITAMD_DEF_EPI(kEpiBiasAddAddRelu, true, 2, 2, fmaxf(((acc + b) + d0) + d1, 0.0f))
+AITAMD_DEF_EPI(kEpiBiasSigmoid, true, 0, 0, sigmoid_f(acc + b))
+AITAMD_DEF_EPI(kEpiBiasTanh, true, 0, 0, tanh_f(acc + b))
+AITAMD_DEF_EPI(kEpiBiasSwish, true, 0, 0, (acc + b) * sigmoid_f(acc + b))
+AITAMD_DEF_EPI(kEpiBiasHardswish, true, 0, 0, hardswish_f(acc + b))
+AITAMD_DEF_EPI(kEpiBiasMul, true, 1, 0, (acc + b) * d0)
+AITAMD_DEF_EPI(kEpiBiasMulAdd, true, 2, 0, (acc + b) * d0 + d1)
+AITAMD_DEF_EPI(kEpiBiasSigmoidMul, true, 1, 0, sigmoid_f(acc + b) * d0)
+AITAMD_DEF_EPI(kEpiBiasSigmoidMulTanh, true, 1, 0, tanh_f(sigmoid_f(acc + b) * d0))
+AITAMD_DEF_EPI(kEpiBiasMulTanh, true, 1, 0, tanh_f((acc + b) * d0))
+AITAMD_DEF_EPI(kEpiAdd, false, 1, 1, acc + d0)
 
 #undef AITAMD_DEF_EPI
+
+// Epi applied to xb = acc (+ bias, already added) and the residuals as stored, with the residual adds that lead
+// the expression folded into the residuals' conversion (see LEAD above).
+template <class Epi, class T>
+AITAMD_DEVICE float apply_folded(float xb, T d0, T d1, float one) {
+  using Tr = ElemTraits<T>;
+  if constexpr (Epi::kLeadingAdds >= 1) xb = Tr::to_float_plus(d0, one, xb);
+  if constexpr (Epi::kLeadingAdds >= 2) xb = Tr::to_float_plus(d1, one, xb);
+  const float f0 = Epi::kLeadingAdds >= 1 ? -0.0f : (Epi::kNumD >= 1 ? Tr::to_float(d0) : 0.0f);
+  const float f1 = Epi::kLeadingAdds >= 2 ? -0.0f : (Epi::kNumD >= 2 ? Tr::to_float(d1) : 0.0f);
+  return Epi::apply(xb, -0.0f, f0, f1);
+}
 
 }  // namespace aitamd

@@ -537,6 +537,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
       vec_ok = vec_ok && ((p.ldd & 1) == 0) && ((p.sd & 1) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 3) == 0);
     if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 3) == 0);
 
+    float one = 1.0f;
+    asm volatile("" : "+s"(one));  // (opaque to the optimizer: see to_float_plus)
     constexpr int PITCH = Tile::EPI_PITCH;
     float* strip = reinterpret_cast<float*>(smem_raw) + wave * MT * PITCH;
     constexpr int LANES_PER_ROW = Tile::WTN / 8;             // lanes covering one strip row
@@ -582,9 +584,11 @@ __global__ void __launch_bounds__(Tile::NT, Tile::OCC) gemm_rcr_dma_kernel(const
             if constexpr (Epi::kNumD >= 2) d1v = *reinterpret_cast<const vec8*>(D1b + d_idx);
             vec8 o;
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-              o[j] = Tr::from_float(
-                  Epi::apply(v[j], Tr::to_float(bv[j]), Tr::to_float(d0v[j]), Tr::to_float(d1v[j])));
+            for (int j = 0; j < 8; ++j) {
+              // bias conversion and add as one instruction where the type has one; -0.0 is the bias that adds nothing
+              const float xb = Epi::kHasBias ? Tr::to_float_plus(bv[j], one, v[j]) : v[j];
+              o[j] = Tr::from_float(apply_folded<Epi, T>(xb, d0v[j], d1v[j], one));
+            }
             store_out(Cb, c_idx, o, p.nt_store != 0, rc);
           } else {
 #pragma unroll

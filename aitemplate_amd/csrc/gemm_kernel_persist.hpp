@@ -21,6 +21,8 @@
 // python/aitemplate/utils/mk_ck_lib/gemm_operation.py:487).
 #pragma once
 
+#include <type_traits>
+
 #include "gemm_kernel_dma.hpp"
 
 
@@ -235,32 +237,32 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       (Epi::kNumD == 0 || (int64_t)BM * p.ldd * 2 < 0x7fffffffll);
   const uint32_t lane_off_c = (uint32_t)((r_row * (int)p.ldc + r_c * 8) * 2);
   const uint32_t lane_off_d = (uint32_t)((r_row * (int)p.ldd + r_c * 8) * 2);
-  auto uniform_ptr = [](const void* ptr) {
-    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
-  };
 
-  auto epilogue_fast = [&](const TileCoord& c) {
+  // NT: cache-policy bits of the stores, a template value so that the choice is made once per tile and the
+  // passes of a strip stay one basic block (math of one pass schedules around the stores of the one before)
+  auto epilogue_fast = [&](const TileCoord& c, auto nt_bits) {
+    constexpr int NT_BITS = decltype(nt_bits)::value;
     const int m_w = c.m0 + wm * Tile::WTM;  // first row and column of the wave's part of the tile
     const int n_w = c.n0 + wn * Tile::WTN;
     const int rows_left = p.M - m_w;
     const uint32_t rows_valid = rows_left <= 0 ? 0u : (uint32_t)(rows_left < Tile::WTM ? rows_left : Tile::WTM);
     T* Cw = reinterpret_cast<T*>(p.c) + out_batch_offset(p, c.batch) + (int64_t)m_w * p.ldc + n_w;
-    const __amdgpu_buffer_rsrc_t rc = make_rsrc(uniform_ptr(Cw), rows_valid * (uint32_t)p.ldc * 2u);
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cw, rows_valid * (uint32_t)p.ldc * 2u);
     __amdgpu_buffer_rsrc_t rd0 = rc, rd1 = rc;
     if constexpr (Epi::kNumD >= 1) {
       const T* Dw = reinterpret_cast<const T*>(p.d0) + (int64_t)c.batch * p.sd + (int64_t)m_w * p.ldd + n_w;
-      rd0 = make_rsrc(uniform_ptr(Dw), rows_valid * (uint32_t)p.ldd * 2u);
+      rd0 = make_rsrc(Dw, rows_valid * (uint32_t)p.ldd * 2u);
     }
     if constexpr (Epi::kNumD >= 2) {
       const T* Dw = reinterpret_cast<const T*>(p.d1) + (int64_t)c.batch * p.sd + (int64_t)m_w * p.ldd + n_w;
-      rd1 = make_rsrc(uniform_ptr(Dw), rows_valid * (uint32_t)p.ldd * 2u);
+      rd1 = make_rsrc(Dw, rows_valid * (uint32_t)p.ldd * 2u);
     }
     const int n = n_w + r_c * 8;  // the lane's 8 columns: the same in every pass
     const bool col_ok = n < p.N;
     const uint32_t off_c0 = col_ok ? lane_off_c : kOobOffset;
     const uint32_t off_d0 = col_ok ? lane_off_d : kOobOffset;
+    float one = 1.0f;
+    asm volatile("" : "+s"(one));  // (opaque to the optimizer: see to_float_plus)
     float bf8[8] = {};
     if constexpr (Epi::kHasBias) {
       if (col_ok) {
@@ -296,15 +298,13 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       for (int ps = 0; ps < Tile::PASSES; ++ps) {
         vec8 o;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          o[j] = Tr::from_float(Epi::apply(Tr::to_float(raw[ps][j]), bf8[j],
-                                           Epi::kNumD >= 1 ? Tr::to_float(d0v[ps][j]) : 0.f,
-                                           Epi::kNumD >= 2 ? Tr::to_float(d1v[ps][j]) : 0.f));
+        for (int j = 0; j < 8; ++j) {
+          // conversion and bias add as one instruction where the type has one; -0.0 is the bias that adds nothing
+          const float xb = Epi::kHasBias ? Tr::to_float_plus(raw[ps][j], one, bf8[j]) : Tr::to_float(raw[ps][j]);
+          o[j] = Tr::from_float(apply_folded<Epi, T>(xb, d0v[ps][j], d1v[ps][j], one));
+        }
         const uint32_t off = off_c0 + (uint32_t)((mi * MT + ps * Tile::ROWS_PER_PASS) * (int)p.ldc * 2);
-        if (p.nt_store)
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, 2);
-        else
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, NT_BITS);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -314,7 +314,10 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   auto epilogue = [&](const TileCoord& c) {
     if (fast_addr) {
-      epilogue_fast(c);
+      if (p.nt_store)
+        epilogue_fast(c, std::integral_constant<int, 2>{});
+      else
+        epilogue_fast(c, std::integral_constant<int, 0>{});
       return;
     }
     T* Cb = reinterpret_cast<T*>(p.c) + out_batch_offset(p, c.batch);
