@@ -40,6 +40,7 @@ constexpr bool kHasPermutedStore = AITAMD_EPI == kEpiNone || AITAMD_EPI == kEpiB
 constexpr int kLayoutBits = (AITAMD_EPI == kEpiNone || AITAMD_EPI == kEpiAdd) ? 0xf : (AITAMD_EPI == kEpiBias ? 0x3 : 0x1);
 constexpr bool kLayoutsArePermuted = AITAMD_EPI == kEpiBias;  // the bias kernels of the other layouts store permuted
 
+constexpr int kShortK = 4;
 template <class Tile, bool PERM, int LAYOUT>
 struct KernelOf {
   static constexpr auto value = gemm_rcr_kernel<Elem, Tile, Epi, PERM, LAYOUT>;
@@ -53,7 +54,9 @@ struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>, P
 
 template <int BM, int BN, int BK, int WM, int WN, int NS, bool PERM, int LAYOUT>
 struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS>, PERM, LAYOUT> {
-  static constexpr auto value = gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS>, Epi, PERM>;
+  // (LAYOUT 4 is not an operand layout: it names the instantiation for tiles of fewer K-slabs than ring stages)
+  static constexpr auto value =
+      gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS>, Epi, PERM, LAYOUT == kShortK>;
 };
 // bit L set: the tile has a kernel for layout L (bit 0, rcr, always)
 template <class Tile>
@@ -185,6 +188,15 @@ hipError_t launch_tile(const GemmParams& p, hipStream_t stream) {
       if (p.layout == 3) return launch_kernel<Tile, kLayoutsArePermuted, 3>(p, stream);
     }
     return hipErrorInvalidValue;
+  }
+  if constexpr (IsPersistent<Tile>::value) {
+    if ((p.K + Tile::BK - 1) / Tile::BK < Tile::NS) {
+      if (p.perm_on) {
+        if constexpr (kHasPermutedStore) return launch_kernel<Tile, true, kShortK>(p, stream);
+        return hipErrorInvalidValue;
+      }
+      return launch_kernel<Tile, false, kShortK>(p, stream);
+    }
   }
   if (p.perm_on) {
     if constexpr (kHasPermutedStore) return launch_kernel<Tile, true>(p, stream);

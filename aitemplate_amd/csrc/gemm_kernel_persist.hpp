@@ -61,7 +61,8 @@ struct GemmTilePersist {
   static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
 };
 
-template <class T, class Tile, class Epi, bool PERM = false>
+// SHORT_K: the instantiation for tiles of fewer K-slabs than ring stages (the launcher picks by K)
+template <class T, class Tile, class Epi, bool PERM = false, bool SHORT_K = false>
 __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const GemmParams p) {
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
@@ -135,9 +136,10 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     return c;
   };
 
-  int ld_i = 0, ld_kt = 0, ld_stage = 0;
-  __amdgpu_buffer_rsrc_t ra, rb;
-  auto set_loader_tile = [&](int i) {
+  // Descriptors of the operand panels of this workgroup's i-th tile.  Past the last tile the ring keeps turning
+  // on zero-sized buffers: every lane is out of range, nothing is fetched, and the number of loads in flight per
+  // step stays constant.
+  auto tile_desc = [&](int i, __amdgpu_buffer_rsrc_t& da, __amdgpu_buffer_rsrc_t& db) {
     if (i < my_tiles) {
       const TileCoord c = tile_coord(i);
       const int rows_a = (p.M - c.m0) < c.rows ? (p.M - c.m0) : c.rows;
@@ -145,22 +147,20 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)c.batch * p.sa + (int64_t)c.m0 * p.lda;
       const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)c.batch * p.sb + (int64_t)c.n0 * p.ldb;
       // (the lower half of a leftover tile can lie wholly below M: nothing to fetch then)
-      ra = make_rsrc(Ab, rows_a > 0 ? clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2) : 0u);
-      rb = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
+      da = make_rsrc(Ab, rows_a > 0 ? clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2) : 0u);
+      db = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
     } else {
-      // past the last tile the ring keeps turning on zero-sized buffers: every lane is out of
-      // range, nothing is fetched, and the number of loads in flight per step stays constant
-      ra = make_rsrc(p.a, 0);
-      rb = make_rsrc(p.b, 0);
+      da = make_rsrc(p.a, 0);
+      db = make_rsrc(p.b, 0);
     }
   };
-  set_loader_tile(0);
 
-  // Issue wave-loads [i0, i1) of the stream's current slab; the portion that ends the slab
-  // advances the stream to the next slab (and tile).
-  auto issue_part = [&](int i0, int i1) {
-    const int k0 = ld_kt * BK;
-    T* sbase = smem + ld_stage * Tile::STAGE_ELEMS;
+  // Issue wave-loads [i0, i1) of K-slab `kt` of the tile behind (da, db) into ring stage `stage`.  No state, no
+  // branches: the slab loop calls it between MFMAs and has to stay one basic block for the interleave to hold.
+  auto issue_part = [&](const __amdgpu_buffer_rsrc_t& da, const __amdgpu_buffer_rsrc_t& db, int kt, int stage, int i0,
+                        int i1) {
+    const int k0 = kt * BK;
+    T* sbase = smem + stage * Tile::STAGE_ELEMS;
 #pragma unroll
     for (int i = 0; i < L; ++i) {
       if (i < i0 || i >= i1) continue;
@@ -169,16 +169,9 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       T* dst = sbase + j * 512;  // 1 KiB per wave-load; A blocks then B blocks
       const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
       if (is_a)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)dst, 16, off, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(da, (lds_void*)dst, 16, off, 0, 0, 0);
       else
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)dst, 16, off, 0, 0, 0);
-    }
-    if (i1 < L) return;
-    ld_stage = ld_stage + 1 == NS ? 0 : ld_stage + 1;
-    if (++ld_kt == k_tiles) {
-      ld_kt = 0;
-      ++ld_i;
-      set_loader_tile(ld_i);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void*)dst, 16, off, 0, 0, 0);
     }
   };
 
@@ -386,54 +379,141 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     }
   };
 
-  // ---- prologue: slabs 0 .. NS-3 whole, slab NS-2 up to its first portion -------------------------
+  // The loader runs ahead of the multiplying: while slab kt of a tile is multiplied, the rest of slab kt + NS - 2
+  // goes out in the slab's first step and the first portion of slab kt + NS - 1 in its last step, into the ring
+  // stage the barrier has just freed.  From slab k_tiles - (NS - 1) on those are slabs of the workgroup's next tile.
+  // Which tile a step loads from is decided by the structure of the code (one slab loop for the bulk of a tile,
+  // NS - 1 peeled slabs for its end), never by a test inside a slab: a conditional there splits the slab into
+  // basic blocks, the loads bunch up behind the barrier instead of alternating with the MFMAs, and the matrix unit
+  // waits for the address unit (measured: 44 us of a 139 us launch).  Needs k_tiles >= NS.
+  constexpr int D1 = NS - 2, D2 = NS - 1;
+  __amdgpu_buffer_rsrc_t ra, rb, nra, nrb;
+  tile_desc(0, ra, rb);
+  if constexpr (SHORT_K) {
+    // Short K: the loader is more than a tile ahead and wraps at places that depend on k_tiles, so it keeps its
+    // position as state and tests for the wrap after every slab it has issued (the conditional costs the
+    // interleave; with so few slabs per tile the epilogue dominates anyway).
+    int ld_i = 0, ld_kt = 0;
+    auto advance = [&]() {
+      if (++ld_kt == k_tiles) {
+        ld_kt = 0;
+        ++ld_i;
+        tile_desc(ld_i, ra, rb);
+      }
+    };
 #pragma unroll
-  for (int s = 0; s < NS - 2; ++s) issue_part(0, L);
-  issue_part(0, L_P0);
+    for (int s = 0; s < NS - 2; ++s) {
+      issue_part(ra, rb, ld_kt, s, 0, L);
+      advance();
+    }
+    issue_part(ra, rb, ld_kt, NS - 2, 0, L_P0);
+    wait_vmcnt<(NS - 3) * L + L_P0>();
+    __builtin_amdgcn_s_barrier();
+    int rd_stage = 0;
+    load_frags(smem, 0, af[0], bf[0]);
+    for (int i = 0; i < my_tiles; ++i) {
+      const TileCoord cur = tile_coord(i);
+      const bool active = wm * Tile::WTM < cur.rows;
+      for (int kt = 0; kt < k_tiles; ++kt) {
+        const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
+        const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
+        const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
+        const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
+        const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
+        issue_part(ra, rb, ld_kt, st1, L_P0, L);
+        advance();
+        if (active) {
+          load_frags(cur_st, 1, af[1], bf[1]);
+          if (kt == 0)
+            mfmas_first(af[0], bf[0]);
+          else
+            mfmas(af[0], bf[0]);
+        }
+        wait_vmcnt<(NS - 3) * L>();
+        __builtin_amdgcn_s_barrier();
+        issue_part(ra, rb, ld_kt, st2, 0, L_P0);
+        if (active) {
+          load_frags(nxt_st, 0, af[0], bf[0]);
+          mfmas(af[1], bf[1]);
+        }
+        rd_stage = nx_stage;
+      }
+      if (active) epilogue(cur);
+    }
+    wait_vmcnt<0>();
+    return;
+  } else {
+  // prologue: slabs 0 .. NS-3 whole, slab NS-2 up to its first portion
+#pragma unroll
+  for (int s = 0; s < NS - 2; ++s) issue_part(ra, rb, s, s, 0, L);
+  issue_part(ra, rb, NS - 2, NS - 2, 0, L_P0);
   wait_vmcnt<(NS - 3) * L + L_P0>();
   __builtin_amdgcn_s_barrier();
   int rd_stage = 0;
   load_frags(smem, 0, af[0], bf[0]);
 
+  // one K-slab: ACTIVE waves multiply, the others only keep the ring turning
+  auto slab = [&](auto active_c, auto first_c, const __amdgpu_buffer_rsrc_t& a1, const __amdgpu_buffer_rsrc_t& b1, int kt1,
+                  const __amdgpu_buffer_rsrc_t& a2, const __amdgpu_buffer_rsrc_t& b2, int kt2) {
+    constexpr bool ACTIVE = decltype(active_c)::value, FIRST = decltype(first_c)::value;
+    const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
+    const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
+    const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
+    const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
+    const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
+    // first step: the rest of the slab whose first portion went out in the previous slab's last step
+    issue_part(a1, b1, kt1, st1, L_P0, L);
+    if constexpr (ACTIVE) {
+      load_frags(cur_st, 1, af[1], bf[1]);
+      if constexpr (FIRST)
+        mfmas_first(af[0], bf[0]);
+      else
+        mfmas(af[0], bf[0]);
+      sched_step<MI * NI, MI + NI, L - L_P0>();
+    }
+    // last step: the next slab has landed once at most (NS-3) younger slabs are in flight; past
+    // the barrier nobody reads the previous slab any more, so its ring slot starts taking a new
+    // slab, and the next slab's first fragments are fetched under this slab's last MFMAs
+    wait_vmcnt<(NS - 3) * L>();
+    __builtin_amdgcn_s_barrier();
+    issue_part(a2, b2, kt2, st2, 0, L_P0);
+    if constexpr (ACTIVE) {
+      load_frags(nxt_st, 0, af[0], bf[0]);
+      mfmas(af[1], bf[1]);
+      sched_step<MI * NI, MI + NI, L_P0>();
+    }
+    rd_stage = nx_stage;
+  };
+  auto tile_slabs = [&](auto active_c) {
+    slab(active_c, std::true_type{}, ra, rb, D1, ra, rb, D2);
+    for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, std::false_type{}, ra, rb, kt + D1, ra, rb, kt + D2);
+#pragma unroll
+    for (int t = 0; t < D2; ++t) {
+      if (t == 0)
+        slab(active_c, std::false_type{}, ra, rb, k_tiles - 1, nra, nrb, 0);
+      else
+        slab(active_c, std::false_type{}, nra, nrb, t - 1, nra, nrb, t);
+    }
+  };
+
   for (int i = 0; i < my_tiles; ++i) {
     const TileCoord cur = tile_coord(i);
+    tile_desc(i + 1, nra, nrb);
     // waves whose rows lie outside a half tile keep the ring turning (their share of the loads, the
     // waits and the barriers) but multiply and store nothing; a half tile is always the last item
     const bool active = wm * Tile::WTM < cur.rows;
-    for (int kt = 0; kt < k_tiles; ++kt) {
-      const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
-      const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
-      const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
-      if (active) {
-        // first step: the rest of the slab whose first portion went out in the previous step
-        issue_part(L_P0, L);
-        load_frags(cur_st, 1, af[1], bf[1]);
-        if (kt == 0)
-          mfmas_first(af[0], bf[0]);
-        else
-          mfmas(af[0], bf[0]);
-        sched_step<MI * NI, MI + NI, L - L_P0>();
-        // last step: the next slab has landed once at most (NS-3) younger slabs are in flight; past
-        // the barrier nobody reads the previous slab any more, so its ring slot starts taking a new
-        // slab, and the next slab's first fragments are fetched under this slab's last MFMAs
-        wait_vmcnt<(NS - 3) * L>();
-        __builtin_amdgcn_s_barrier();
-        issue_part(0, L_P0);
-        load_frags(nxt_st, 0, af[0], bf[0]);
-        mfmas(af[1], bf[1]);
-        sched_step<MI * NI, MI + NI, L_P0>();
-      } else {
-        issue_part(L_P0, L);
-        wait_vmcnt<(NS - 3) * L>();
-        __builtin_amdgcn_s_barrier();
-        issue_part(0, L_P0);
-      }
-      rd_stage = nx_stage;
+    if (active) {
+      tile_slabs(std::true_type{});
+      epilogue(cur);
+    } else {
+      tile_slabs(std::false_type{});
     }
-    if (active) epilogue(cur);
+    ra = nra;
+    rb = nrb;
   }
   // no LDS-DMA may be in flight into a workgroup that has ended
   wait_vmcnt<0>();
+  }
 }
 
 }  // namespace aitamd
