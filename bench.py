@@ -265,8 +265,11 @@ def cpu_baseline(torch, max_seconds=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    # defaults: the first 200 or so launches after an idle spell run up to 1.5x slower (clocks and translation
+    # caches settle over some 30 ms); 500 untimed launches put the timed region into the steady state a loaded
+    # server is in
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--algo", default="-1",
                     help="kernel instance, by index or by name (default: see --select)")
     ap.add_argument("--select", choices=("profile", "heuristic"), default="profile",
@@ -341,7 +344,7 @@ def main():
     }
     del case
     if not args.no_other_configs:
-        line["other_configs"] = other_configs(torch, eager, _kernels, max(20, args.steps // 2), max(5, args.warmup // 2))
+        line["other_configs"] = other_configs(torch, eager, _kernels, max(20, min(200, args.steps // 2)), max(5, min(50, args.warmup // 2)))
     if not args.no_in_abi:
         line["in_abi"] = in_abi(torch)
     if not args.no_cpu_baseline:
