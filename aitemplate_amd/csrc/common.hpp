@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace aitamd {
 
 using f16 = _Float16;
@@ -91,6 +93,16 @@ AITAMD_DEVICE typename ElemTraits<T>::vec8 join_halves(typename ElemTraits<T>::v
 // Raw buffer resources.  Loads whose byte offset is >= num_records return 0,
 // which is how every M/N/K tail is zero-filled without branches.
 // ---------------------------------------------------------------------------
+// f(integral_constant<int, I>) for I in [I0, I1): a loop whose index is a constant expression in the body
+// (immediate operands of builtins)
+template <int I0, int I1, class F>
+AITAMD_DEVICE void static_for(F&& f) {
+  if constexpr (I0 < I1) {
+    f(std::integral_constant<int, I0>{});
+    static_for<I0 + 1, I1>(f);
+  }
+}
+
 constexpr uint32_t kOobOffset = 0x80000000u;  // >= any num_records we build
 
 // Every descriptor in these kernels is the same for all lanes of a wave (one per tile, batch entry or wave

@@ -104,18 +104,24 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   const int my_tiles = full_rounds + (split ? (split_tile < left ? 1 : 0) : (g < left ? 1 : 0));
 
   // ---- loader: a stream of slabs that runs across this workgroup's tiles ------------------------
+  // A ring stage holds A_LOADS + B_LOADS blocks of 1 KiB (ROWS_PER_LOAD rows of a slab each, A then B); a wave
+  // fetches the L consecutive blocks wave * L ... with one direct-to-LDS load each, so it reads only A or only B.
+  // The loads of one portion ([0, L_P0) or [L_P0, L)) share one LDS base: the instruction's immediate offset
+  // places the later ones (it shifts the global address as well, which the lane offsets take back).  Writing
+  // the LDS base register before every load instead costs a fifth of the whole kernel's time.
+  static_assert(Tile::A_LOADS % L == 0, "a wave's blocks must not straddle A and B");
+  const bool loads_a = wave * L < Tile::A_LOADS;
   const int l_row = lane / Tile::CPR;
   const int l_slot = lane % Tile::CPR;
   uint32_t l_off[L];
   int l_chunk_k[L];
 #pragma unroll
   for (int i = 0; i < L; ++i) {
-    const int j = wave + i * Tile::NW;
-    // (with A_LOADS a multiple of the wave count, whether load i fetches A or B is the same for every wave)
-    const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
-    const int row = (is_a ? j : j - Tile::A_LOADS) * Tile::ROWS_PER_LOAD + l_row;
+    const int j = wave * L + i;
+    const int row = (loads_a ? j : j - Tile::A_LOADS) * Tile::ROWS_PER_LOAD + l_row;
     const int chunk = l_slot ^ ((row / Tile::RPW) % Tile::CPR);
-    l_off[i] = (uint32_t)(((int64_t)row * (is_a ? p.lda : p.ldb) + chunk * 8) * 2);
+    const int in_portion = SHORT_K ? 0 : (i < L_P0 ? i : i - L_P0);
+    l_off[i] = (uint32_t)(((int64_t)row * (loads_a ? p.lda : p.ldb) + chunk * 8) * 2 - in_portion * 1024);
     l_chunk_k[i] = chunk * 8;
   }
 
@@ -136,10 +142,10 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     return c;
   };
 
-  // Descriptors of the operand panels of this workgroup's i-th tile.  Past the last tile the ring keeps turning
-  // on zero-sized buffers: every lane is out of range, nothing is fetched, and the number of loads in flight per
-  // step stays constant.
-  auto tile_desc = [&](int i, __amdgpu_buffer_rsrc_t& da, __amdgpu_buffer_rsrc_t& db) {
+  // Descriptor of the operand panel (A or B) this wave fetches for the workgroup's i-th tile.  Past the last tile
+  // the ring keeps turning on a zero-sized buffer: every lane is out of range, nothing is fetched, and the number
+  // of loads in flight per step stays constant.
+  auto tile_desc = [&](int i, __amdgpu_buffer_rsrc_t& d) {
     if (i < my_tiles) {
       const TileCoord c = tile_coord(i);
       const int rows_a = (p.M - c.m0) < c.rows ? (p.M - c.m0) : c.rows;
@@ -147,32 +153,28 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)c.batch * p.sa + (int64_t)c.m0 * p.lda;
       const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)c.batch * p.sb + (int64_t)c.n0 * p.ldb;
       // (the lower half of a leftover tile can lie wholly below M: nothing to fetch then)
-      da = make_rsrc(Ab, rows_a > 0 ? clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2) : 0u);
-      db = make_rsrc(Bb, clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2));
+      const uint32_t bytes_a = rows_a > 0 ? clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2) : 0u;
+      const uint32_t bytes_b = clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2);
+      d = make_rsrc(loads_a ? Ab : Bb, loads_a ? bytes_a : bytes_b);
     } else {
-      da = make_rsrc(p.a, 0);
-      db = make_rsrc(p.b, 0);
+      d = make_rsrc(p.a, 0);
     }
   };
 
-  // Issue wave-loads [i0, i1) of K-slab `kt` of the tile behind (da, db) into ring stage `stage`.  No state, no
+  // Issue wave-loads [I0, I1) of K-slab `kt` of the tile behind `d` into ring stage `stage`.  No state, no
   // branches: the slab loop calls it between MFMAs and has to stay one basic block for the interleave to hold.
-  auto issue_part = [&](const __amdgpu_buffer_rsrc_t& da, const __amdgpu_buffer_rsrc_t& db, int kt, int stage, int i0,
-                        int i1) {
+  auto issue_part = [&](auto i0_c, auto i1_c, const __amdgpu_buffer_rsrc_t& d, int kt, int stage) {
+    constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
     const int k0 = kt * BK;
-    T* sbase = smem + stage * Tile::STAGE_ELEMS;
-#pragma unroll
-    for (int i = 0; i < L; ++i) {
-      if (i < i0 || i >= i1) continue;
-      const int j = wave + i * Tile::NW;
+    T* dst = smem + stage * Tile::STAGE_ELEMS + (wave * L + I0) * 512;  // 1 KiB per wave-load
+    static_for<I0, I1>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
       const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + (uint32_t)(k0 * 2) : kOobOffset;
-      T* dst = sbase + j * 512;  // 1 KiB per wave-load; A blocks then B blocks
-      const bool is_a = Tile::A_LOADS % Tile::NW == 0 ? i * Tile::NW < Tile::A_LOADS : j < Tile::A_LOADS;
-      if (is_a)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(da, (lds_void*)dst, 16, off, 0, 0, 0);
+      if constexpr (SHORT_K)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (lds_void*)(dst + (i - I0) * 512), 16, off, 0, 0, 0);
       else
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(db, (lds_void*)dst, 16, off, 0, 0, 0);
-    }
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (lds_void*)dst, 16, off, 0, (i - I0) * 1024, 0);
+    });
   };
 
   // ---- fragments ------------------------------------------------------------------------------
@@ -387,8 +389,12 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   // basic blocks, the loads bunch up behind the barrier instead of alternating with the MFMAs, and the matrix unit
   // waits for the address unit (measured: 44 us of a 139 us launch).  Needs k_tiles >= NS.
   constexpr int D1 = NS - 2, D2 = NS - 1;
-  __amdgpu_buffer_rsrc_t ra, rb, nra, nrb;
-  tile_desc(0, ra, rb);
+  constexpr std::integral_constant<int, 0> c_0{};
+  constexpr std::integral_constant<int, L_P0> c_P{};
+  constexpr std::integral_constant<int, L> c_L{};
+  static_assert(L_P0 > 0 && L_P0 < L, "a slab goes out in two portions");
+  __amdgpu_buffer_rsrc_t rd, nrd;  // this wave's operand panel of the current and of the next tile
+  tile_desc(0, rd);
   if constexpr (SHORT_K) {
     // Short K: the loader is more than a tile ahead and wraps at places that depend on k_tiles, so it keeps its
     // position as state and tests for the wrap after every slab it has issued (the conditional costs the
@@ -398,15 +404,16 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       if (++ld_kt == k_tiles) {
         ld_kt = 0;
         ++ld_i;
-        tile_desc(ld_i, ra, rb);
+        tile_desc(ld_i, rd);
       }
     };
 #pragma unroll
     for (int s = 0; s < NS - 2; ++s) {
-      issue_part(ra, rb, ld_kt, s, 0, L);
+      issue_part(c_0, c_P, rd, ld_kt, s);
+      issue_part(c_P, c_L, rd, ld_kt, s);
       advance();
     }
-    issue_part(ra, rb, ld_kt, NS - 2, 0, L_P0);
+    issue_part(c_0, c_P, rd, ld_kt, NS - 2);
     wait_vmcnt<(NS - 3) * L + L_P0>();
     __builtin_amdgcn_s_barrier();
     int rd_stage = 0;
@@ -420,7 +427,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
         const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
         const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
-        issue_part(ra, rb, ld_kt, st1, L_P0, L);
+        issue_part(c_P, c_L, rd, ld_kt, st1);
         advance();
         if (active) {
           load_frags(cur_st, 1, af[1], bf[1]);
@@ -431,7 +438,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         }
         wait_vmcnt<(NS - 3) * L>();
         __builtin_amdgcn_s_barrier();
-        issue_part(ra, rb, ld_kt, st2, 0, L_P0);
+        issue_part(c_0, c_P, rd, ld_kt, st2);
         if (active) {
           load_frags(nxt_st, 0, af[0], bf[0]);
           mfmas(af[1], bf[1]);
@@ -445,16 +452,20 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   } else {
   // prologue: slabs 0 .. NS-3 whole, slab NS-2 up to its first portion
 #pragma unroll
-  for (int s = 0; s < NS - 2; ++s) issue_part(ra, rb, s, s, 0, L);
-  issue_part(ra, rb, NS - 2, NS - 2, 0, L_P0);
+  for (int s = 0; s < NS - 2; ++s) {
+    // (portion by portion: the lane offsets assume the immediate offsets of a portion's loads)
+    issue_part(c_0, c_P, rd, s, s);
+    issue_part(c_P, c_L, rd, s, s);
+  }
+  issue_part(c_0, c_P, rd, NS - 2, NS - 2);
   wait_vmcnt<(NS - 3) * L + L_P0>();
   __builtin_amdgcn_s_barrier();
   int rd_stage = 0;
   load_frags(smem, 0, af[0], bf[0]);
 
   // one K-slab: ACTIVE waves multiply, the others only keep the ring turning
-  auto slab = [&](auto active_c, auto first_c, const __amdgpu_buffer_rsrc_t& a1, const __amdgpu_buffer_rsrc_t& b1, int kt1,
-                  const __amdgpu_buffer_rsrc_t& a2, const __amdgpu_buffer_rsrc_t& b2, int kt2) {
+  auto slab = [&](auto active_c, auto first_c, const __amdgpu_buffer_rsrc_t& d1, int kt1,
+                  const __amdgpu_buffer_rsrc_t& d2, int kt2) {
     constexpr bool ACTIVE = decltype(active_c)::value, FIRST = decltype(first_c)::value;
     const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
     const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
@@ -462,7 +473,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
     const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
     // first step: the rest of the slab whose first portion went out in the previous slab's last step
-    issue_part(a1, b1, kt1, st1, L_P0, L);
+    issue_part(c_P, c_L, d1, kt1, st1);
     if constexpr (ACTIVE) {
       load_frags(cur_st, 1, af[1], bf[1]);
       if constexpr (FIRST)
@@ -476,7 +487,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     // slab, and the next slab's first fragments are fetched under this slab's last MFMAs
     wait_vmcnt<(NS - 3) * L>();
     __builtin_amdgcn_s_barrier();
-    issue_part(a2, b2, kt2, st2, 0, L_P0);
+    issue_part(c_0, c_P, d2, kt2, st2);
     if constexpr (ACTIVE) {
       load_frags(nxt_st, 0, af[0], bf[0]);
       mfmas(af[1], bf[1]);
@@ -485,20 +496,20 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     rd_stage = nx_stage;
   };
   auto tile_slabs = [&](auto active_c) {
-    slab(active_c, std::true_type{}, ra, rb, D1, ra, rb, D2);
-    for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, std::false_type{}, ra, rb, kt + D1, ra, rb, kt + D2);
+    slab(active_c, std::true_type{}, rd, D1, rd, D2);
+    for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, std::false_type{}, rd, kt + D1, rd, kt + D2);
 #pragma unroll
     for (int t = 0; t < D2; ++t) {
       if (t == 0)
-        slab(active_c, std::false_type{}, ra, rb, k_tiles - 1, nra, nrb, 0);
+        slab(active_c, std::false_type{}, rd, k_tiles - 1, nrd, 0);
       else
-        slab(active_c, std::false_type{}, nra, nrb, t - 1, nra, nrb, t);
+        slab(active_c, std::false_type{}, nrd, t - 1, nrd, t);
     }
   };
 
   for (int i = 0; i < my_tiles; ++i) {
     const TileCoord cur = tile_coord(i);
-    tile_desc(i + 1, nra, nrb);
+    tile_desc(i + 1, nrd);
     // waves whose rows lie outside a half tile keep the ring turning (their share of the loads, the
     // waits and the barriers) but multiply and store nothing; a half tile is always the last item
     const bool active = wm * Tile::WTM < cur.rows;
@@ -508,8 +519,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     } else {
       tile_slabs(std::false_type{});
     }
-    ra = nra;
-    rb = nrb;
+    rd = nrd;
   }
   // no LDS-DMA may be in flight into a workgroup that has ended
   wait_vmcnt<0>();
