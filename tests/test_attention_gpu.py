@@ -222,3 +222,62 @@ def test_nan_in_a_key_gives_nan_for_its_batch_entry_only():
         for g in range(G):
             if keep[bo, g]:
                 torch.testing.assert_close(got[bo, :, g, :], want[bo, :, g, :], atol=TOL, rtol=TOL)
+
+
+# ---- head dims 16 KS - 8 (24, 40, 56, 88, 120, 152) in fp16 take the form that folds the scale and the softmax's
+# reference point into the first product (a 1 in K's first padding column against -m in Q's); everything the plain
+# form is tested for has to hold there too
+@pytest.mark.parametrize("B,M,N,K,O,G,causal,scale", [
+    (8, 300, 700, 40, 40, 4, False, None),
+    (8, 300, 300, 40, 40, 4, True, None),
+    (4, 130, 1000, 40, 64, 2, False, -0.2),     # negative scale: changes sides into Q
+    (6, 64, 77, 24, 24, 3, False, None),
+    (6, 200, 200, 24, 32, 3, True, None),
+    (4, 100, 520, 56, 56, 2, False, None),
+    (4, 257, 257, 88, 88, 2, True, None),
+    (2, 96, 300, 120, 120, 2, False, None),
+    (2, 64, 200, 152, 152, 1, False, None),
+])
+def test_folded_form_head_dims(B, M, N, K, O, G, causal, scale):
+    _check(B, M, N, K, O, G, causal, scale=scale, seed=K + M)
+
+
+def test_folded_form_large_and_small_logits():
+    """The folded form rounds Q |scale| log2(e) to fp16: the error of a logit is 2^-11 of its terms' magnitude.  Pins
+    the envelope: logits up to about 100 stay within the 2e-2 tolerance (the plain form, which bf16 keeps, is exact in
+    the scale), rows whose scores are all far below zero do not underflow to a zero sum, and tiny logits are exact."""
+    B, M, N, K, G = 8, 256, 600, 40, 4
+    for mult, shift, tol in ((4.0, 0.0, 2e-2), (1.0, -30.0, 2e-2), (0.01, 0.0, 2e-3)):
+        print(f"case attention folded logits x{mult} shift {shift}", flush=True)
+        q, k, v = _rand((B, M, K), torch.float16, 31) * mult, _rand((B, N, K), torch.float16, 32) * mult, \
+            _rand((B, N, K), torch.float16, 33)
+        if shift:
+            # every score of a row about `shift`: q gets a constant component that k answers with a negative one
+            q[..., 0] = 8.0
+            k[..., 0] = shift / 8.0 * K ** 0.5
+        want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, K ** -0.5, G, False).half().float()
+        got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
+        assert torch.isfinite(got).all()
+        torch.testing.assert_close(got, want, atol=tol, rtol=tol)
+    # bf16 keeps the plain form: large logits stay accurate there (3e-2 is the bf16 tolerance of the other tests)
+    q, k, v = _rand((B, M, K), torch.bfloat16, 34) * 4, _rand((B, N, K), torch.bfloat16, 35) * 4, \
+        _rand((B, N, K), torch.bfloat16, 36)
+    want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, K ** -0.5, G, False).bfloat16().float()
+    got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
+    torch.testing.assert_close(got, want, atol=3e-2, rtol=3e-2)
+
+
+def test_folded_form_nan_key_and_lengths(attn_variant):
+    """NaN propagation and the length masks at head dim 40 (the folded form's own masked and unmasked blocks)."""
+    B, M, N, K, O, G = 4, 96, 200, 40, 40, 2
+    q, k, v = _rand((B, M, K), torch.float16, 41), _rand((B, N, K), torch.float16, 42), _rand((B, N, O), torch.float16, 43)
+    k[1, 77, 5] = float("nan")
+    want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, K ** -0.5, G, False).half().float()
+    got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
+    assert torch.isnan(got[0, :, 1, :]).all() and torch.isnan(want[0, :, 1, :]).all()
+    for bo, g in ((0, 0), (1, 0), (1, 1)):
+        torch.testing.assert_close(got[bo, :, g, :], want[bo, :, g, :], atol=TOL, rtol=TOL)
+    for mode in (-1, 0, 1, 2, 3):
+        attn_variant(mode)
+        _check_mem_eff(3, 4, 150, 333, 40, 40, [333, 1, 200], causal=False)
+        _check_mem_eff(3, 4, 150, 150, 40, 40, [150, 0, 77], causal=True, lens_q=[150, 10, 0])
