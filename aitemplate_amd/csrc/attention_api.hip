@@ -68,19 +68,10 @@ struct TileOf<KS, OT, 3> {
   using type = AttnTile<KS, OT, Base::BN, 4, kFits ? 4 : 2, kFits ? 2 : 1>;
 };
 
-template <class T, int KS, int OT, bool VEC, bool DMA, int MODE, bool FOLD = false>
+template <class T, int KS, int OT, bool VEC, bool DMA, int MODE>
 hipError_t launch_attention(const AttnParams& p, hipStream_t stream) {
-  constexpr bool FOLD_OK = !FOLD;  // (the folded launcher does not dispatch again)
   using Tile = typename TileOf<KS, OT, MODE>::type;
-  // head dim 16 KS - 8 on the vector paths: the form that folds scale and reference point into the first product
-  // (fp16 only: the folded form rounds Q |scale| log2(e) to the element type, an error of 2^-11 of a logit's
-  // magnitude per term - under 2e-2 in the output up to logits of about 100; bf16's 2^-8 is too coarse for that.
-  // AITAMD_ATTN_FOLD=0, read once, keeps fp16 on the exact form as well.)
-  if constexpr (VEC && DMA && FOLD_OK && std::is_same<T, f16>::value) {
-    static const bool fold_on = !(getenv("AITAMD_ATTN_FOLD") && atoi(getenv("AITAMD_ATTN_FOLD")) == 0);
-    if (fold_on && p.K == 16 * KS - 8) return launch_attention<T, KS, OT, VEC, DMA, MODE, true>(p, stream);
-  }
-  auto kernel = attention_kernel<T, Tile, VEC, DMA, FOLD>;
+  auto kernel = attention_kernel<T, Tile, VEC, DMA>;
   static std::once_flag once[kMaxDevices];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);

@@ -162,15 +162,9 @@ AITAMD_DEVICE void attn_wait_vmcnt_upto(int n) {
   }
 }
 
-// FOLD (head dim K = 16 KS - 8, e.g. 40): the scale and the softmax's reference point ride in the first product.
-// Q is multiplied by |scale| log2(e) when its fragments are built, the first of the eight padding columns of K reads
-// 1 and the same column of Q holds -m, so the matrix unit delivers s c - m and a probability costs one v_exp
-// instead of an FMA and a v_exp.  m is a value of the element type (it is an operand); it moves, as in the plain
-// form, only when a row's maximum has outgrown it by 2^kLazyLog2, and then that block subtracts the step by hand.
-template <class T, class Tile, bool VEC, bool DMA = false, bool FOLD = false>
+template <class T, class Tile, bool VEC, bool DMA = false>
 __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_kernel(const AttnParams p) {
   static_assert(!DMA || VEC, "the direct-to-LDS path needs 16-byte chunks");
-  static_assert(!FOLD || VEC, "the folded form needs K to be whole 16-byte chunks");
   static_assert(DMA || Tile::NS == 2, "the register-staged loaders double-buffer");
   static_assert(DMA || Tile::NG == 1, "wave groups need the direct-to-LDS loader");
   constexpr int NS = Tile::NS, NW = Tile::NW, NG = Tile::NG, NWT = NW * NG;
@@ -246,16 +240,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = -v[j];
       }
-      if constexpr (FOLD) {
-        const float cq = __builtin_fabsf(p.scale_log2e);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = Tr::from_float(Tr::to_float(v[j]) * cq);
-      }
       qf[ks] = v;
     }
-    // FOLD: lanes h = 1 of the last fragment hold the padding columns K .. K + 7; column K is the one that carries
-    // the reference point (0 until a row has seen a live key) against a 1 in K's fragment
-    const uint32_t k_one = (FOLD && h == 1) ? (uint32_t)__builtin_bit_cast(uint16_t, Tr::from_float(1.0f)) : 0u;
 
     // ---- tile loaders: global -> registers -> LDS, zero-filled past N / K / O
     u32x4 kreg[Tile::K_IT], vreg[Tile::V_IT];
@@ -446,15 +432,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           for (int e = 0; e < 16; ++e) s[kb][e] = 0.0f;
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
-            vec8 kf =
+            const vec8 kf =
                 *reinterpret_cast<const vec8*>(cK + ((blk * KB + kb) * 32 + r32) * KPI + ks * 16 + h * 8);
-            if constexpr (FOLD) {
-              if (ks == KS - 1) {
-                u32x4 kw = __builtin_bit_cast(u32x4, kf);
-                kw[0] |= k_one;  // (the padding columns are zero-filled by the loaders)
-                kf = __builtin_bit_cast(vec8, kw);
-              }
-            }
             s[kb] = Tr::mfma32(kf, qf[ks], s[kb]);
           }
         }
@@ -484,38 +463,6 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
 #pragma unroll
             for (int e = 0; e < 16; ++e) text = fmaxf(text, (MASKED && dead[kb][e]) ? -INFINITY : s[kb][e]);
           text = max_across_halves(text);
-          if constexpr (FOLD) {
-            // s holds s c - m already (s c while the row has no reference point yet)
-            constexpr float kLazyLog2 = 8.0f;
-            const bool first = __builtin_isinf(m_run);
-            const bool move = first ? (text > -INFINITY) : (text > kLazyLog2);
-            const float base = first ? 0.0f : m_run;
-            const float m_new = move ? Tr::to_float(Tr::from_float(base + text)) : m_run;
-            const float shift = move ? m_new - base : 0.0f;
-            alpha = !move ? 1.0f : (first ? 0.0f : __builtin_amdgcn_exp2f(-shift));
-            l_run *= alpha;
-            // wave-uniform: the block in which some row's reference point moves pays the subtraction, the others
-            // (most of them) exponentiate the product as it comes
-            auto probabilities = [&](auto shifted_tag) {
-#pragma unroll
-              for (int st = 0; st < 2 * KB; ++st) {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                  const int kb = st >> 1, e = (st & 1) * 8 + j;
-                  const float x = decltype(shifted_tag)::value ? s[kb][e] - shift : s[kb][e];
-                  pf[st][j] = Tr::from_float((MASKED && dead[kb][e]) ? 0.0f : __builtin_amdgcn_exp2f(x));
-                }
-                l_run = add_elements(pf[st], l_run);
-              }
-            };
-            if (__builtin_amdgcn_ballot_w64(move) != 0)
-              probabilities(std::true_type{});
-            else
-              probabilities(std::false_type{});
-            m_run = m_new;
-            if (h == 1) qf[KS - 1][0] = Tr::from_float(__builtin_isinf(m_run) ? 0.0f : -m_run);
-            return;
-          }
           const float m_cand = fmaxf(m_run, text);
           // The reference point of the exponent moves only when the row maximum has grown by more than
           // kLazyLog2 binary orders since it was last taken: until then p = exp2(s c - m c) may exceed 1 (by at
@@ -601,9 +548,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         const float l1 = xch[((NV - 1) * NW + wave) * 64 + lane];
         // both states are sums of exp2((s - m) c) terms for their own reference m: bring them to the larger one
         const float m = fmaxf(m_run, m1);
-        const float cm = FOLD ? 1.0f : c;  // (FOLD keeps m in units of the exponent)
-        const float a0 = __builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m) * cm);
-        const float a1 = __builtin_isinf(m1) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * cm);
+        const float a0 = __builtin_isinf(m_run) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m) * c);
+        const float a1 = __builtin_isinf(m1) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * c);
         l_run = l_run * a0 + l1 * a1;
 #pragma unroll
         for (int ot = 0; ot < OT; ++ot)

@@ -224,9 +224,7 @@ def test_nan_in_a_key_gives_nan_for_its_batch_entry_only():
                 torch.testing.assert_close(got[bo, :, g, :], want[bo, :, g, :], atol=TOL, rtol=TOL)
 
 
-# ---- head dims 16 KS - 8 (24, 40, 56, 88, 120, 152) in fp16 take the form that folds the scale and the softmax's
-# reference point into the first product (a 1 in K's first padding column against -m in Q's); everything the plain
-# form is tested for has to hold there too
+# ---- head dims that leave padding columns in the LDS tiles (K = 16 KS - 8: 24, 40, 56, 88, 120, 152; O = 32 OT - 24)
 @pytest.mark.parametrize("B,M,N,K,O,G,causal,scale", [
     (8, 300, 700, 40, 40, 4, False, None),
     (8, 300, 300, 40, 40, 4, True, None),
@@ -237,18 +235,24 @@ def test_nan_in_a_key_gives_nan_for_its_batch_entry_only():
     (4, 257, 257, 88, 88, 2, True, None),
     (2, 96, 300, 120, 120, 2, False, None),
     (2, 64, 200, 152, 152, 1, False, None),
+    # K = 16 KS - 8 with O = 32 OT - 24
+    (6, 100, 333, 24, 8, 3, False, None),
+    (4, 200, 520, 56, 40, 2, True, None),
+    (4, 130, 300, 88, 72, 2, False, None),
+    (2, 96, 260, 120, 104, 2, True, None),
+    (2, 64, 200, 152, 136, 1, False, None),
+    (70000, 8, 40, 40, 40, 7, False, None),    # more batch entries than the grid's y range: a workgroup takes two
 ])
-def test_folded_form_head_dims(B, M, N, K, O, G, causal, scale):
+def test_head_dims_with_padding_columns(B, M, N, K, O, G, causal, scale):
     _check(B, M, N, K, O, G, causal, scale=scale, seed=K + M)
 
 
-def test_folded_form_large_and_small_logits():
-    """The folded form rounds Q |scale| log2(e) to fp16: the error of a logit is 2^-11 of its terms' magnitude.  Pins
-    the envelope: logits up to about 100 stay within the 2e-2 tolerance (the plain form, which bf16 keeps, is exact in
-    the scale), rows whose scores are all far below zero do not underflow to a zero sum, and tiny logits are exact."""
+def test_large_small_and_all_negative_logits():
+    """Logits of about 100 (a sharply peaked softmax), rows whose scores are all far below zero (the running maximum
+    must not start at 0: the sum would underflow) and tiny logits; fp16 and bf16."""
     B, M, N, K, G = 8, 256, 600, 40, 4
     for mult, shift, tol in ((4.0, 0.0, 2e-2), (1.0, -30.0, 2e-2), (0.01, 0.0, 2e-3)):
-        print(f"case attention folded logits x{mult} shift {shift}", flush=True)
+        print(f"case attention logits x{mult} shift {shift}", flush=True)
         q, k, v = _rand((B, M, K), torch.float16, 31) * mult, _rand((B, N, K), torch.float16, 32) * mult, \
             _rand((B, N, K), torch.float16, 33)
         if shift:
@@ -259,7 +263,7 @@ def test_folded_form_large_and_small_logits():
         got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
         assert torch.isfinite(got).all()
         torch.testing.assert_close(got, want, atol=tol, rtol=tol)
-    # bf16 keeps the plain form: large logits stay accurate there (3e-2 is the bf16 tolerance of the other tests)
+    # (3e-2 is the bf16 tolerance of the other tests)
     q, k, v = _rand((B, M, K), torch.bfloat16, 34) * 4, _rand((B, N, K), torch.bfloat16, 35) * 4, \
         _rand((B, N, K), torch.bfloat16, 36)
     want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, K ** -0.5, G, False).bfloat16().float()
@@ -267,8 +271,8 @@ def test_folded_form_large_and_small_logits():
     torch.testing.assert_close(got, want, atol=3e-2, rtol=3e-2)
 
 
-def test_folded_form_nan_key_and_lengths(attn_variant):
-    """NaN propagation and the length masks at head dim 40 (the folded form's own masked and unmasked blocks)."""
+def test_nan_key_and_lengths_at_head_dim_40(attn_variant):
+    """NaN propagation and the length masks at head dim 40 (padded to 48 / 64 inside LDS), every variant."""
     B, M, N, K, O, G = 4, 96, 200, 40, 40, 2
     q, k, v = _rand((B, M, K), torch.float16, 41), _rand((B, N, K), torch.float16, 42), _rand((B, N, O), torch.float16, 43)
     k[1, 77, 5] = float("nan")
