@@ -28,9 +28,14 @@
 
 namespace aitamd {
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_>
+// MT_: edge of the MFMA's output block.  32: v_mfma_f32_32x32x16, two K-steps per 32-deep slab.  16:
+// v_mfma_f32_16x16x32, one K-step per slab, whose blocks are multiplied in two halves (upper and lower block rows)
+// around the slab's barrier; the 16x16x32 form moves half the accumulator registers per multiply-add and sustains
+// 13 % more under the board's power limit on random operands (1.93 against 1.71 PFLOP/s in a loop of MFMAs alone).
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int MT_ = 32>
 struct GemmTilePersist {
-  static constexpr int MT = 32, KSTEP = 16, QN = 2, ACC_N = 16;
+  static constexpr int MT = MT_, KSTEP = MT == 32 ? 16 : 32, QN = 64 / MT, ACC_N = MT * MT / 64;
+  static constexpr int SB = 32;  // rows of an epilogue strip pass (one or two block rows)
   static constexpr int BM = BM_, BN = BN_, BK = BK_;
   static constexpr int WGM = WGM_, WGN = WGN_, NS = NS_;
   static constexpr int NW = WGM * WGN;
@@ -50,11 +55,13 @@ struct GemmTilePersist {
   // wave-private epilogue strip: 32 rows x WTN elements of the output type
   static constexpr int STRIP_CHUNKS = WTN / 8;  // 16-byte chunks per strip row
   static constexpr int STRIP_PITCH = WTN * 2;
-  static constexpr int STRIP_BYTES = MT * STRIP_PITCH;
+  static constexpr int STRIP_BYTES = SB * STRIP_PITCH;
   static constexpr int ROWS_PER_PASS = 64 / STRIP_CHUNKS;
-  static constexpr int PASSES = MT / ROWS_PER_PASS;
+  static constexpr int PASSES = SB / ROWS_PER_PASS;
   static constexpr int kLdsBytes = RING_BYTES + NW * STRIP_BYTES;
-  static_assert(KK == 2, "two MFMA steps per slab");
+  static_assert(MT == 32 || MT == 16, "MFMA block is 32x32 or 16x16");
+  static_assert((MT == 32 && KK == 2) || (MT == 16 && KK == 1 && MI % 2 == 0), "a slab is multiplied in two halves");
+  static_assert(WTM % SB == 0, "a wave's rows are whole strip passes");
   static_assert(NS >= 4, "needs one slab in flight behind the one being waited for");
   static_assert((A_LOADS + B_LOADS) % NW == 0, "slab loads must divide over the waves");
   static_assert(STRIP_CHUNKS == 4 || STRIP_CHUNKS == 8 || STRIP_CHUNKS == 16, "strip swizzle needs 2^k chunks");
@@ -66,10 +73,11 @@ template <class T, class Tile, class Epi, bool PERM = false, bool SHORT_K = fals
 __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const GemmParams p) {
   using Tr = ElemTraits<T>;
   using vec8 = typename Tr::vec8;
-  using Mfma = MfmaOp<T, 32>;
+  using Mfma = MfmaOp<T, Tile::MT>;
   using acc_t = typename Mfma::acc_t;
   constexpr int BM = Tile::BM, BN = Tile::BN, BK = Tile::BK, NS = Tile::NS;
-  constexpr int MI = Tile::MI, NI = Tile::NI, MT = 32;
+  constexpr int MI = Tile::MI, NI = Tile::NI, MT = Tile::MT, KK = Tile::KK, QN = Tile::QN, SB = Tile::SB;
+  constexpr int MH = KK == 1 ? MI / 2 : MI;  // block rows multiplied per half of a slab
   constexpr int L = Tile::LOADS_PER_STEP, L_P0 = Tile::L_P0;
   constexpr int SC = Tile::STRIP_CHUNKS;
   typedef __attribute__((address_space(3))) void lds_void;
@@ -82,8 +90,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Tile::WGN;
   const int wn = wave % Tile::WGN;
-  const int fr = lane & 31;
-  const int fq = lane >> 5;
+  const int fr = lane % MT;
+  const int fq = lane / MT;
   unsigned char* const strip = smem_raw + Tile::RING_BYTES + wave * Tile::STRIP_BYTES;
 
   const int tiles_per_batch = p.tiles_m * p.tiles_n;
@@ -178,34 +186,82 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   };
 
   // ---- fragments ------------------------------------------------------------------------------
-  int a_rd[2], b_rd[2];
+  int a_rd[KK], b_rd[KK];
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk) {
-    a_rd[kk] = dma_lds_chunk_elem<Tile>(wm * Tile::WTM + fr, kk * 2 + fq);
-    b_rd[kk] = BM * BK + dma_lds_chunk_elem<Tile>(wn * Tile::WTN + fr, kk * 2 + fq);
+  for (int kk = 0; kk < KK; ++kk) {
+    a_rd[kk] = dma_lds_chunk_elem<Tile>(wm * Tile::WTM + fr, kk * QN + fq);
+    b_rd[kk] = BM * BK + dma_lds_chunk_elem<Tile>(wn * Tile::WTN + fr, kk * QN + fq);
   }
-  auto load_frags = [&](const T* st, int kk, vec8* af, vec8* bf) {
+  // KK == 2: half `hh` of a slab is K-step hh over all block rows (af[hh][0 .. MI), bf[hh][0 .. NI)).
+  // KK == 1: half `hh` is block rows hh * MH ... of the one K-step (af[hh][0 .. MH)); both halves use bf[0].
+  auto load_a = [&](const T* st, int hh, vec8* af) {
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[kk] + mi * MT * BK);
+    for (int mi = 0; mi < MH; ++mi)
+      af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[KK == 1 ? 0 : hh] + ((KK == 1 ? hh * MH : 0) + mi) * MT * BK);
+  };
+  auto load_b1 = [&](const T* st, int hh, int ni) {
+    return *reinterpret_cast<const vec8*>(st + b_rd[KK == 1 ? 0 : hh] + ni * MT * BK);
+  };
+  auto load_frags = [&](const T* st, int hh, vec8* af, vec8* bf) {
+    load_a(st, hh, af);
 #pragma unroll
-    for (int ni = 0; ni < NI; ++ni) bf[ni] = *reinterpret_cast<const vec8*>(st + b_rd[kk] + ni * MT * BK);
+    for (int ni = 0; ni < NI; ++ni) bf[ni] = load_b1(st, hh, ni);
   };
   acc_t acc[MI][NI];
-  vec8 af[2][MI], bf[2][NI];
+  vec8 af[2][MH], bf[KK][NI];
   // operands swapped: the MFMA produces the transposed block, so a lane holds 4 consecutive
   // output columns of one row
-  auto mfmas = [&](const vec8* a, const vec8* b) {
+  // (m0: first block row of the half: 0, or MH for the lower half of a one-step slab)
+  auto mfmas = [&](const vec8* a, const vec8* b, int m0 = 0) {
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
+    for (int mi = 0; mi < MH; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = Mfma::run(b[ni], a[mi], acc[mi][ni]);
+      for (int ni = 0; ni < NI; ++ni) acc[m0 + mi][ni] = Mfma::run(b[ni], a[mi], acc[m0 + mi][ni]);
   };
-  auto mfmas_first = [&](const vec8* a, const vec8* b) {
+  auto mfmas_first = [&](const vec8* a, const vec8* b, int m0 = 0) {
     const acc_t zero = {};
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
+    for (int mi = 0; mi < MH; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = Mfma::run(b[ni], a[mi], zero);
+      for (int ni = 0; ni < NI; ++ni) acc[m0 + mi][ni] = Mfma::run(b[ni], a[mi], zero);
+  };
+
+  // The two halves of a slab.  The first fetches what the second needs and multiplies K-step 0 (the upper block
+  // rows of a one-step slab); the second multiplies the rest and fetches the first half of the next slab.  With
+  // one K-step per slab the B fragments serve both halves and are single-buffered: each is replaced by the next
+  // slab's as soon as the MFMAs of its block column have been issued.
+  auto half1_reads = [&](const T* cur_st) {
+    if constexpr (KK == 2)
+      load_frags(cur_st, 1, af[1], bf[1]);
+    else
+      load_a(cur_st, 1, af[1]);
+  };
+  auto half1_mfmas = [&](auto first_c) {
+    if constexpr (decltype(first_c)::value)
+      mfmas_first(af[0], bf[0]);
+    else
+      mfmas(af[0], bf[0]);
+  };
+  auto half2_reads = [&](const T* nxt_st) {
+    if constexpr (KK == 2)
+      load_frags(nxt_st, 0, af[0], bf[0]);
+    else
+      load_a(nxt_st, 0, af[0]);
+  };
+  auto half2_mfmas = [&](auto first_c, const T* nxt_st) {
+    constexpr bool FIRST = decltype(first_c)::value;
+    if constexpr (KK == 2) {
+      mfmas(af[1], bf[1]);
+    } else {
+      const acc_t zero = {};
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+        for (int mi = 0; mi < MH; ++mi)
+          acc[MH + mi][ni] = Mfma::run(bf[0][ni], af[1][mi], FIRST ? zero : acc[MH + mi][ni]);
+        bf[0][ni] = load_b1(nxt_st, 0, ni);
+      }
+    }
   };
 
   // ---- epilogue -------------------------------------------------------------------------------
@@ -219,10 +275,30 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     vec_ok = vec_ok && ((p.ldd & 1) == 0) && ((p.sd & 1) == 0) && ((reinterpret_cast<uintptr_t>(p.d0) & 3) == 0);
   if (Epi::kNumD >= 2) vec_ok = vec_ok && ((reinterpret_cast<uintptr_t>(p.d1) & 3) == 0);
   // strip addressing: row r, 16-byte chunk c lives at r * PITCH + ((c ^ (r % SC)) << 4)
-  const int w_base = fr * Tile::STRIP_PITCH + fq * 8;
-  const int w_swz = fr & (SC - 1);
   const int r_row = lane / SC;
   const int r_c = lane % SC;
+  // Strip block `sb` (SB = 32 rows of the wave's part: one block row of 32x32 MFMAs, two of 16x16) goes to the
+  // strip in the output type.  A lane holds, per MFMA block and group g, 4 consecutive columns
+  // ni * MT + g * 4 QN + 4 fq of row fr.
+  auto write_strip = [&](int sb) {
+    constexpr int SUB = SB / MT;       // block rows per strip block
+    constexpr int NG = Tile::ACC_N / 4;
+#pragma unroll
+    for (int sub = 0; sub < SUB; ++sub) {
+      const int row = sub * MT + fr;
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int gq = 0; gq < NG; ++gq) {
+          typename Tr::vec4 h;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) h[j] = Tr::from_float(acc[sb * SUB + sub][ni][gq * 4 + j]);
+          const int col = ni * MT + gq * (QN * 4) + fq * 4;
+          *reinterpret_cast<u32x2*>(strip + row * Tile::STRIP_PITCH + (((col >> 3) ^ (row & (SC - 1))) << 4) +
+                                    (col & 7) * 2) = __builtin_bit_cast(u32x2, h);
+        }
+    }
+  };
 
   // Fast form of the epilogue's addressing (plain store, N a multiple of 8, a tile's rows span less than
   // 2 GiB): the output and the residuals are addressed through buffer descriptors that start at the wave's
@@ -267,16 +343,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       }
     }
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
-#pragma unroll
-      for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          typename Tr::vec4 h;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) h[j] = Tr::from_float(acc[mi][ni][gq * 4 + j]);
-          *reinterpret_cast<u32x2*>(strip + w_base + (((ni * 4 + gq) ^ w_swz) << 4)) = __builtin_bit_cast(u32x2, h);
-        }
+    for (int sb = 0; sb < Tile::WTM / SB; ++sb) {
+      write_strip(sb);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -285,7 +353,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       for (int ps = 0; ps < Tile::PASSES; ++ps) {
         const int row = ps * Tile::ROWS_PER_PASS + r_row;
         raw[ps] = *reinterpret_cast<const vec8*>(strip + row * Tile::STRIP_PITCH + ((r_c ^ (row & (SC - 1))) << 4));
-        const uint32_t step_d = (uint32_t)((mi * MT + ps * Tile::ROWS_PER_PASS) * (int)p.ldd * 2);
+        const uint32_t step_d = (uint32_t)((sb * SB + ps * Tile::ROWS_PER_PASS) * (int)p.ldd * 2);
         if constexpr (Epi::kNumD >= 1) d0v[ps] = __builtin_bit_cast(vec8, buffer_load_16B(rd0, off_d0 + step_d));
         if constexpr (Epi::kNumD >= 2) d1v[ps] = __builtin_bit_cast(vec8, buffer_load_16B(rd1, off_d0 + step_d));
       }
@@ -298,7 +366,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
           const float xb = Epi::kHasBias ? Tr::to_float_plus(raw[ps][j], one, bf8[j]) : Tr::to_float(raw[ps][j]);
           o[j] = Tr::from_float(apply_folded<Epi, T>(xb, d0v[ps][j], d1v[ps][j], one));
         }
-        const uint32_t off = off_c0 + (uint32_t)((mi * MT + ps * Tile::ROWS_PER_PASS) * (int)p.ldc * 2);
+        const uint32_t off = off_c0 + (uint32_t)((sb * SB + ps * Tile::ROWS_PER_PASS) * (int)p.ldc * 2);
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, NT_BITS);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -329,16 +397,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       }
     }
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
-#pragma unroll
-      for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          typename Tr::vec4 h;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) h[j] = Tr::from_float(acc[mi][ni][gq * 4 + j]);
-          *reinterpret_cast<u32x2*>(strip + w_base + (((ni * 4 + gq) ^ w_swz) << 4)) = __builtin_bit_cast(u32x2, h);
-        }
+    for (int sb = 0; sb < Tile::WTM / SB; ++sb) {
+      write_strip(sb);
       // the strip is private to the wave and LDS executes one wave's accesses in order
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -348,7 +408,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         const int row = ps * Tile::ROWS_PER_PASS + r_row;
         const vec8 raw =
             *reinterpret_cast<const vec8*>(strip + row * Tile::STRIP_PITCH + ((r_c ^ (row & (SC - 1))) << 4));
-        const int m = c.m0 + wm * Tile::WTM + mi * MT + row;
+        const int m = c.m0 + wm * Tile::WTM + sb * SB + row;
         if (m < p.M && n < p.N) {
           const int64_t c_idx = out_index<PERM>(p, m, n);
           const int64_t d_idx = (int64_t)m * p.ldd + n;
@@ -430,18 +490,21 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         issue_part(c_P, c_L, rd, ld_kt, st1);
         advance();
         if (active) {
-          load_frags(cur_st, 1, af[1], bf[1]);
+          half1_reads(cur_st);
           if (kt == 0)
-            mfmas_first(af[0], bf[0]);
+            half1_mfmas(std::true_type{});
           else
-            mfmas(af[0], bf[0]);
+            half1_mfmas(std::false_type{});
         }
         wait_vmcnt<(NS - 3) * L>();
         __builtin_amdgcn_s_barrier();
         issue_part(c_0, c_P, rd, ld_kt, st2);
         if (active) {
-          load_frags(nxt_st, 0, af[0], bf[0]);
-          mfmas(af[1], bf[1]);
+          half2_reads(nxt_st);
+          if (kt == 0)
+            half2_mfmas(std::true_type{}, nxt_st);
+          else
+            half2_mfmas(std::false_type{}, nxt_st);
         }
         rd_stage = nx_stage;
       }
@@ -473,14 +536,12 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
     const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
     // first step: the rest of the slab whose first portion went out in the previous slab's last step
+    // first step: the rest of the slab whose first portion went out in the previous slab's last step
     issue_part(c_P, c_L, d1, kt1, st1);
     if constexpr (ACTIVE) {
-      load_frags(cur_st, 1, af[1], bf[1]);
-      if constexpr (FIRST)
-        mfmas_first(af[0], bf[0]);
-      else
-        mfmas(af[0], bf[0]);
-      sched_step<MI * NI, MI + NI, L - L_P0>();
+      half1_reads(cur_st);
+      half1_mfmas(first_c);
+      if constexpr (KK == 2) sched_step<MI * NI, MI + NI, L - L_P0>();
     }
     // last step: the next slab has landed once at most (NS-3) younger slabs are in flight; past
     // the barrier nobody reads the previous slab any more, so its ring slot starts taking a new
@@ -489,9 +550,11 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     __builtin_amdgcn_s_barrier();
     issue_part(c_0, c_P, d2, kt2, st2);
     if constexpr (ACTIVE) {
-      load_frags(nxt_st, 0, af[0], bf[0]);
-      mfmas(af[1], bf[1]);
-      sched_step<MI * NI, MI + NI, L_P0>();
+      half2_reads(nxt_st);
+      half2_mfmas(first_c, nxt_st);
+      // (one-step slabs take no scheduling hints: reads in pairs behind the first MFMAs and loads spread over
+      // the rest, the order the hints give two-step slabs, ran 3 to 5 % slower there than the compiler's own)
+      if constexpr (KK == 2) sched_step<MI * NI, MI + NI, L_P0>();
     }
     rd_stage = nx_stage;
   };

@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 # same counter read for the 256 MiB copy of --copy-probe in the same run).  An instance that is not listed was
 # never measured and reports null with that reason.
 MEASURED_TRAFFIC = {
-    "gemm_rcr_f16_256x256x32_w2x4_persist4": (331_326_000, "profiles/gemm_rcr_persist_kernel_bias_gelu_M24576_N3072_K768_counters.txt"),
+    "gemm_rcr_f16_256x256x32_w2x4_persist4_m16": (331_326_000, "profiles/gemm_rcr_persist_kernel_bias_gelu_M24576_N3072_K768_counters.txt"),
 }
 
 SHAPES = {
