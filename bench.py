@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 # same counter read for the 256 MiB copy of --copy-probe in the same run).  An instance that is not listed was
 # never measured and reports null with that reason.
 MEASURED_TRAFFIC = {
-    "gemm_rcr_f16_256x256x32_w2x4_persist4_m16": (331_326_000, "profiles/gemm_rcr_persist_kernel_bias_gelu_M24576_N3072_K768_counters.txt"),
+    "gemm_rcr_f16_256x256x32_w2x4_persist4_m16": (331_374_000, "profiles/gemm_rcr_persist_kernel_bias_gelu_M24576_N3072_K768_counters.txt"),
 }
 
 SHAPES = {
@@ -49,7 +49,59 @@ def _median(values):
     return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
 
 
-def timed_region(torch, step, steps, warmup, groups=20, graph=False):
+class PowerSampler:
+    """Board power from the amdgpu hwmon files of the first card, read every 20 ms by a thread while a timed
+    region runs.  Reports nothing (None) where the files are missing or unreadable."""
+
+    def __init__(self):
+        import glob
+        self.path = self.cap_path = None
+        for h in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+            for f in ("power1_average", "power1_input"):
+                if os.path.exists(os.path.join(h, f)):
+                    self.path = os.path.join(h, f)
+                    self.cap_path = os.path.join(h, "power1_cap")
+                    break
+            if self.path:
+                break
+        self.samples = []
+
+    def _read(self, path):
+        try:
+            with open(path) as f:
+                return int(f.read()) / 1e6
+        except (OSError, ValueError, TypeError):
+            return None
+
+    def __enter__(self):
+        import threading
+        self.samples = []
+        self._stop = threading.Event()
+
+        def loop():
+            while not self._stop.is_set():
+                w = self._read(self.path) if self.path else None
+                if w is not None:
+                    self.samples.append(w)
+                self._stop.wait(0.02)
+        self._thread = threading.Thread(target=loop, daemon=True)
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join()
+
+    def report(self):
+        if not self.samples:
+            return None
+        cap = self._read(self.cap_path) if self.cap_path else None
+        tail = self.samples[len(self.samples) * 2 // 5:]  # the sensor averages over about a second: drop the ramp
+        return {"avg_w": round(sum(tail) / len(tail), 1), "max_w": round(max(tail), 1), "cap_w": cap, "samples": len(tail),
+                "source": f"{os.path.basename(self.path)} of the card's hwmon, every 20 ms over the last 60 % of the region"}
+
+
+def timed_region(torch, step, steps, warmup, groups=20, graph=False, power=None):
     """W untimed steps, then exactly K steps between two device synchronisations.  Events on the launch stream
     bracket the region and cut it into up to `groups` groups of consecutive launches: the region's average and
     the median of the group averages both come from the same K launches.  With `graph` the K steps are captured
@@ -75,6 +127,8 @@ def timed_region(torch, step, steps, warmup, groups=20, graph=False):
         cuts = [per * k for k in range(groups + 1)]
         steps = per * groups
     events = [torch.cuda.Event(enable_timing=True) for _ in cuts]
+    if power is not None:
+        power.__enter__()
     t0 = time.perf_counter()
     events[0].record()
     for k in range(groups):
@@ -86,6 +140,8 @@ def timed_region(torch, step, steps, warmup, groups=20, graph=False):
         events[k + 1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
+    if power is not None:
+        power.__exit__()
     per_group = [events[k].elapsed_time(events[k + 1]) / (cuts[k + 1] - cuts[k]) for k in range(groups)]
     return {"steps": steps, "wall_ms_per_step": wall_ms / steps,
             "event_ms_per_launch": events[0].elapsed_time(events[-1]) / steps,
@@ -198,6 +254,35 @@ def other_configs(torch, eager, kernels, steps, warmup):
     return out
 
 
+def power_and_vendor_baseline(torch, eager, case, algo, seconds=2.5):
+    """Board power under the headline launch, and a baseline that is not part of the product: the bias-only GEMM of
+    the headline shape through this library and through torch.nn.functional.linear (the vendor's GEMM library under
+    PyTorch-ROCm; it has no fused tanh-GELU epilogue, so the comparison is on gemm_rcr_bias).  Each leg repeats its
+    launch for about `seconds`, long enough for the board's power sensor, on the same rotating operand sets, one
+    leg after the other in this process."""
+    pool, out = case.pool, {}
+
+    def ours_bias(i):
+        x, w, b, _, o = pool[i % len(pool)]
+        eager.gemm("gemm_rcr_bias", x, w, b, out=o)
+
+    def vendor(i):
+        x, w, b, _, o = pool[i % len(pool)]
+        torch.nn.functional.linear(x, w, b)
+    for name, fn in (("headline_launch", case.step_fn(algo)), ("this_library_gemm_rcr_bias", ours_bias),
+                     ("torch_nn_functional_linear", vendor)):
+        try:
+            ps = PowerSampler()
+            r = timed_region(torch, fn, int(seconds / 0.000125), 300, power=ps)
+            out[name] = {"median_ms": round(r["median_ms_per_launch"], 5),
+                         "tflops": round(case.flops / r["median_ms_per_launch"] / 1e9, 2), "board_power": ps.report()}
+        except Exception as e:  # a baseline must never take the bench line down
+            out[name] = {"error": f"{type(e).__name__}: {e}"}
+    out["note"] = (f"M={case.M} N={case.N} K={case.K} fp16, {int(seconds / 0.000125)} launches per leg after 300 untimed; "
+                   "headline_launch is gemm_rcr_bias_gelu, the other two are gemm_rcr_bias")
+    return out
+
+
 def copy_probe(torch, nbytes=256 << 20, reps=5):
     """A plain device copy of known size, for scaling the FETCH_SIZE / WRITE_SIZE counters of a
     counter-collection run of this script (the copy reads nbytes and writes nbytes per launch)."""
@@ -283,6 +368,9 @@ def main():
     ap.add_argument("--no-constant-data", action="store_true",
                     help="skip the diagnostic launch of the same kernel on constant operands")
     ap.add_argument("--no-in-abi", action="store_true", help="skip the compile_model + container Benchmark leg")
+    ap.add_argument("--no-vendor-baseline", action="store_true",
+                    help="skip the board-power legs (headline launch, bias-only GEMM through this library and through "
+                         "torch.nn.functional.linear)")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="time the headline configuration only (for profiler runs of one kernel)")
     args = ap.parse_args()
@@ -366,6 +454,8 @@ def main():
                    "instance_selected_by": "--algo" if algo_given else args.select},
         "roofline": roofline,
     }
+    if not args.no_vendor_baseline:
+        line["power_and_vendor_baseline"] = power_and_vendor_baseline(torch, eager, case, algo)
     del case
     if not args.no_other_configs:
         line["other_configs"] = other_configs(torch, eager, _kernels, max(20, min(200, args.steps // 2)), max(5, min(50, args.warmup // 2)))
