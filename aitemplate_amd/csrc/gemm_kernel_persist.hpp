@@ -116,6 +116,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   const int split_half = (g >> 3) & 1;
   const int my_tiles = full_rounds + (split ? (split_tile < left ? 1 : 0) : (g < left ? 1 : 0));
 
+  // (Every lambda below is force-inlined: left to its size heuristics the compiler has kept the slab lambda of a
+  // four-wave instantiation as a real function, with the accumulators passed through scratch memory.)
   // ---- loader: a stream of slabs that runs across this workgroup's tiles ------------------------
   // A ring stage holds A_LOADS + B_LOADS blocks of 1 KiB (ROWS_PER_LOAD rows of a slab each, A then B); a wave
   // fetches the L consecutive blocks wave * L ... with one direct-to-LDS load each, so it reads only A or only B.
@@ -142,7 +144,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     int m0, n0, batch;
     int rows;  // rows of the tile this workgroup computes: BM, or BM / 2 for half a leftover tile
   };
-  auto tile_coord = [&](int i) {
+  auto tile_coord = [&](int i) __attribute__((always_inline)) {
     TileCoord c;
     // virtual workgroup index: with one workgroup per CU, g % 8 is the XCD and stays it for every i
     int b, tm, tn;
@@ -158,7 +160,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   // Descriptor of the operand panel (A or B) this wave fetches for the workgroup's i-th tile.  Past the last tile
   // the ring keeps turning on a zero-sized buffer: every lane is out of range, nothing is fetched, and the number
   // of loads in flight per step stays constant.
-  auto tile_desc = [&](int i, __amdgpu_buffer_rsrc_t& d) {
+  auto tile_desc = [&](int i, __amdgpu_buffer_rsrc_t& d) __attribute__((always_inline)) {
     if (i < my_tiles) {
       const TileCoord c = tile_coord(i);
       const int rows_a = (p.M - c.m0) < c.rows ? (p.M - c.m0) : c.rows;
@@ -176,7 +178,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   // Issue wave-loads [I0, I1) of K-slab `kt` of the tile behind `d` into ring stage `stage`.  No state, no
   // branches: the slab loop calls it between MFMAs and has to stay one basic block for the interleave to hold.
-  auto issue_part = [&](auto i0_c, auto i1_c, const __amdgpu_buffer_rsrc_t& d, int kt, int stage) {
+  auto issue_part = [&](auto i0_c, auto i1_c, const __amdgpu_buffer_rsrc_t& d, int kt, int stage) __attribute__((always_inline)) {
     constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
     const int k0 = kt * BK;
     T* dst = smem + stage * Tile::STAGE_ELEMS + (wave * L + I0) * 512;  // 1 KiB per wave-load
@@ -199,15 +201,15 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   }
   // KK == 2: half `hh` of a slab is K-step hh over all block rows (af[hh][0 .. MI), bf[hh][0 .. NI)).
   // KK == 1: half `hh` is block rows hh * MH ... of the one K-step (af[hh][0 .. MH)); both halves use bf[0].
-  auto load_a = [&](const T* st, int hh, vec8* af) {
+  auto load_a = [&](const T* st, int hh, vec8* af) __attribute__((always_inline)) {
 #pragma unroll
     for (int mi = 0; mi < MH; ++mi)
       af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[KK == 1 ? 0 : hh] + ((KK == 1 ? hh * MH : 0) + mi) * MT * BK);
   };
-  auto load_b1 = [&](const T* st, int hh, int ni) {
+  auto load_b1 = [&](const T* st, int hh, int ni) __attribute__((always_inline)) {
     return *reinterpret_cast<const vec8*>(st + b_rd[KK == 1 ? 0 : hh] + ni * MT * BK);
   };
-  auto load_frags = [&](const T* st, int hh, vec8* af, vec8* bf) {
+  auto load_frags = [&](const T* st, int hh, vec8* af, vec8* bf) __attribute__((always_inline)) {
     load_a(st, hh, af);
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) bf[ni] = load_b1(st, hh, ni);
@@ -217,13 +219,13 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   // operands swapped: the MFMA produces the transposed block, so a lane holds 4 consecutive
   // output columns of one row
   // (m0: first block row of the half: 0, or MH for the lower half of a one-step slab)
-  auto mfmas = [&](const vec8* a, const vec8* b, int m0 = 0) {
+  auto mfmas = [&](const vec8* a, const vec8* b, int m0 = 0) __attribute__((always_inline)) {
 #pragma unroll
     for (int mi = 0; mi < MH; ++mi)
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) acc[m0 + mi][ni] = Mfma::run(b[ni], a[mi], acc[m0 + mi][ni]);
   };
-  auto mfmas_first = [&](const vec8* a, const vec8* b, int m0 = 0) {
+  auto mfmas_first = [&](const vec8* a, const vec8* b, int m0 = 0) __attribute__((always_inline)) {
     const acc_t zero = {};
 #pragma unroll
     for (int mi = 0; mi < MH; ++mi)
@@ -235,25 +237,25 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   // rows of a one-step slab); the second multiplies the rest and fetches the first half of the next slab.  With
   // one K-step per slab the B fragments serve both halves and are single-buffered: each is replaced by the next
   // slab's as soon as the MFMAs of its block column have been issued.
-  auto half1_reads = [&](const T* cur_st) {
+  auto half1_reads = [&](const T* cur_st) __attribute__((always_inline)) {
     if constexpr (KK == 2)
       load_frags(cur_st, 1, af[1], bf[1]);
     else
       load_a(cur_st, 1, af[1]);
   };
-  auto half1_mfmas = [&](auto first_c) {
+  auto half1_mfmas = [&](auto first_c) __attribute__((always_inline)) {
     if constexpr (decltype(first_c)::value)
       mfmas_first(af[0], bf[0]);
     else
       mfmas(af[0], bf[0]);
   };
-  auto half2_reads = [&](const T* nxt_st) {
+  auto half2_reads = [&](const T* nxt_st) __attribute__((always_inline)) {
     if constexpr (KK == 2)
       load_frags(nxt_st, 0, af[0], bf[0]);
     else
       load_a(nxt_st, 0, af[0]);
   };
-  auto half2_mfmas = [&](auto first_c, const T* nxt_st) {
+  auto half2_mfmas = [&](auto first_c, const T* nxt_st) __attribute__((always_inline)) {
     constexpr bool FIRST = decltype(first_c)::value;
     if constexpr (KK == 2) {
       mfmas(af[1], bf[1]);
@@ -285,7 +287,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   // Strip block `sb` (SB = 32 rows of the wave's part: one block row of 32x32 MFMAs, two of 16x16) goes to the
   // strip in the output type.  A lane holds, per MFMA block and group g, 4 consecutive columns
   // ni * MT + g * 4 QN + 4 fq of row fr.
-  auto write_strip = [&](int sb) {
+  auto write_strip = [&](int sb) __attribute__((always_inline)) {
     constexpr int SUB = SB / MT;       // block rows per strip block
     constexpr int NG = Tile::ACC_N / 4;
 #pragma unroll
@@ -316,7 +318,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   // NT: cache-policy bits of the stores, a template value so that the choice is made once per tile and the
   // passes of a strip stay one basic block (math of one pass schedules around the stores of the one before)
-  auto epilogue_fast = [&](const TileCoord& c, auto nt_bits) {
+  auto epilogue_fast = [&](const TileCoord& c, auto nt_bits) __attribute__((always_inline)) {
     constexpr int NT_BITS = decltype(nt_bits)::value;
     const int m_w = c.m0 + wm * Tile::WTM;  // first row and column of the wave's part of the tile
     const int n_w = c.n0 + wn * Tile::WTN;
@@ -380,7 +382,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     }
   };
 
-  auto epilogue = [&](const TileCoord& c) {
+  auto epilogue = [&](const TileCoord& c) __attribute__((always_inline)) {
     if (fast_addr) {
       if (p.nt_store)
         epilogue_fast(c, std::integral_constant<int, 2>{});
@@ -465,7 +467,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     // position as state and tests for the wrap after every slab it has issued (the conditional costs the
     // interleave; with so few slabs per tile the epilogue dominates anyway).
     int ld_i = 0, ld_kt = 0;
-    auto advance = [&]() {
+    auto advance = [&]() __attribute__((always_inline)) {
       if (++ld_kt == k_tiles) {
         ld_kt = 0;
         ++ld_i;
@@ -533,7 +535,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 
   // one K-slab: ACTIVE waves multiply, the others only keep the ring turning
   auto slab = [&](auto active_c, auto first_c, const __amdgpu_buffer_rsrc_t& d1, int kt1,
-                  const __amdgpu_buffer_rsrc_t& d2, int kt2) {
+                  const __amdgpu_buffer_rsrc_t& d2, int kt2) __attribute__((always_inline)) {
     constexpr bool ACTIVE = decltype(active_c)::value, FIRST = decltype(first_c)::value;
     const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
     const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
@@ -563,7 +565,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     }
     rd_stage = nx_stage;
   };
-  auto tile_slabs = [&](auto active_c) {
+  auto tile_slabs = [&](auto active_c) __attribute__((always_inline)) {
     slab(active_c, std::true_type{}, rd, D1, rd, D2);
     for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, std::false_type{}, rd, kt + D1, rd, kt + D2);
 #pragma unroll
