@@ -14,7 +14,8 @@
 //
 // Epilogue: the accumulators are rounded to the output type, transposed through a
 // wave-private LDS strip outside the ring (32 rows at a time, 16-byte chunks XOR-
-// swizzled, conflict-free both ways), read back as 8 consecutive columns per lane,
+// swizzled: the 16-byte reads are free of bank conflicts, the 8-byte writes take 1.3
+// times the conflict-free time), read back as 8 consecutive columns per lane,
 // combined with bias / residuals in fp32 and stored with 16-byte stores.  Rounding
 // the accumulator before the element-wise functor is what the reference's
 // Composable-Kernel path does too (C-shuffle to the C type, then the functor;
