@@ -217,7 +217,7 @@ def _roofline(bound, work, ms_avg, ms_median):
             "frac": round(achieved / peak, 4), "frac_at_median_launch": round(work / ms_median / scale / peak, 4)}
 
 
-def other_configs(torch, eager, kernels, steps, warmup):
+def other_configs(torch, eager, kernels, steps, warmup, vendor_baseline=True):
     """Configurations 1, 2b, 3 (MFMA-bound GEMMs), 4 (bmm_rcr, HBM-bound) and 5 (fused attention)."""
     out = {}
     for name in ("c1", "c2b", "c3"):
@@ -251,6 +251,15 @@ def other_configs(torch, eager, kernels, steps, warmup):
                  "ms": round(r5["event_ms_per_launch"], 5), "median_ms": round(r5["median_ms_per_launch"], 5),
                  "tflops": round(f5 / r5["event_ms_per_launch"] / 1e9, 2),
                  "roofline": _roofline("mfma", f5, r5["event_ms_per_launch"], r5["median_ms_per_launch"])}
+    if vendor_baseline:
+        # a baseline, not part of the product: PyTorch-ROCm's fused attention on the same operand sets
+        try:
+            sdpa = torch.nn.functional.scaled_dot_product_attention
+            v5 = [tuple(t.view(2, 8, 4096, 40) for t in s) for s in sets5]
+            rv = timed_region(torch, lambda i: sdpa(*v5[i % 16]), steps, warmup)
+            out["c5"]["vendor_baseline"] = {"torch_scaled_dot_product_attention_median_ms": round(rv["median_ms_per_launch"], 5)}
+        except Exception as e:
+            out["c5"]["vendor_baseline"] = {"error": f"{type(e).__name__}: {e}"}
     return out
 
 
@@ -458,7 +467,8 @@ def main():
         line["power_and_vendor_baseline"] = power_and_vendor_baseline(torch, eager, case, algo)
     del case
     if not args.no_other_configs:
-        line["other_configs"] = other_configs(torch, eager, _kernels, max(20, min(200, args.steps // 2)), max(5, min(50, args.warmup // 2)))
+        line["other_configs"] = other_configs(torch, eager, _kernels, max(20, min(200, args.steps // 2)), max(5, min(50, args.warmup // 2)),
+                                              vendor_baseline=not args.no_vendor_baseline)
     if not args.no_in_abi:
         line["in_abi"] = in_abi(torch)
     if not args.no_cpu_baseline:
