@@ -231,6 +231,23 @@ def other_configs(torch, eager, kernels, steps, warmup, vendor_baseline=True):
                      "ms": round(r["event_ms_per_launch"], 5), "median_ms": round(r["median_ms_per_launch"], 5),
                      "tflops": round(case.flops / r["event_ms_per_launch"] / 1e9, 2),
                      "roofline": _roofline("mfma", case.flops, r["event_ms_per_launch"], r["median_ms_per_launch"])}
+        if vendor_baseline:
+            # a baseline, not part of the product: the same result from PyTorch-ROCm's own operators on the same
+            # operand sets (its GEMM library with a bias, then one add kernel per residual)
+            try:
+                pool, nres = case.pool, case.nres
+
+                def torch_ops(i):
+                    x, w, b, d, _ = pool[i % len(pool)]
+                    y = torch.nn.functional.linear(x, w, b)
+                    for t in d[:nres]:
+                        y = y + t
+                    return y
+                rv = timed_region(torch, torch_ops, steps, warmup, graph=graph)
+                out[name]["vendor_baseline"] = {"torch_linear_plus_adds_median_ms": round(rv["median_ms_per_launch"], 5),
+                                                "kernels_per_step": 1 + nres}
+            except Exception as e:
+                out[name]["vendor_baseline"] = {"error": f"{type(e).__name__}: {e}"}
         del case
     g = torch.Generator(device="cuda").manual_seed(4)
     sets4 = [(torch.randn(768, 384, 64, device="cuda", generator=g).half() / 8,
@@ -241,6 +258,13 @@ def other_configs(torch, eager, kernels, steps, warmup, vendor_baseline=True):
     out["c4"] = {"op": "bmm_rcr", "B": 768, "M": 384, "N": 384, "K": 64, "ms": round(r4["event_ms_per_launch"], 5),
                  "median_ms": round(r4["median_ms_per_launch"], 5),
                  "roofline": _roofline("hbm", b4, r4["event_ms_per_launch"], r4["median_ms_per_launch"])}
+    if vendor_baseline:
+        try:
+            rv = timed_region(torch, lambda i: torch.bmm(sets4[i % 3][0], sets4[i % 3][1].transpose(1, 2), out=sets4[i % 3][2]),
+                              steps, warmup)
+            out["c4"]["vendor_baseline"] = {"torch_bmm_median_ms": round(rv["median_ms_per_launch"], 5)}
+        except Exception as e:
+            out["c4"]["vendor_baseline"] = {"error": f"{type(e).__name__}: {e}"}
     del sets4
     sets5 = [tuple(torch.randn(16, 4096, 40, device="cuda", generator=g).half() for _ in range(3)) for _ in range(16)]
     out5 = torch.empty(2, 4096, 8, 40, device="cuda", dtype=torch.float16)
