@@ -1,0 +1,54 @@
+"""Host-side pieces of bench.py that need no GPU: the argument contract and the power-sensor reader."""
+import os
+import subprocess
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+import bench  # noqa: E402
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr
+
+
+def test_median():
+    assert bench._median([3.0, 1.0, 2.0]) == 2.0
+    assert bench._median([4.0, 1.0, 2.0, 3.0]) == 2.5
+
+
+def test_power_sampler_reads_microwatts_and_drops_the_ramp(tmp_path):
+    power, cap = tmp_path / "power1_input", tmp_path / "power1_cap"
+    power.write_text("250000000\n")
+    cap.write_text("1400000000\n")
+    ps = bench.PowerSampler()
+    ps.path, ps.cap_path = str(power), str(cap)
+    with ps:
+        time.sleep(0.15)
+        power.write_text("1380000000\n")
+        time.sleep(0.3)
+    rep = ps.report()
+    assert rep["cap_w"] == 1400.0
+    assert rep["max_w"] == 1380.0
+    assert rep["avg_w"] > 1000.0  # the first two fifths of the samples are not counted
+    assert rep["samples"] >= 5
+
+
+def test_power_sampler_without_a_sensor_reports_nothing(tmp_path):
+    ps = bench.PowerSampler()
+    ps.path, ps.cap_path = str(tmp_path / "missing"), None
+    with ps:
+        time.sleep(0.05)
+    assert ps.report() is None
+
+
+def test_traffic_table_names_files_that_exist():
+    for instance, (nbytes, path) in bench.MEASURED_TRAFFIC.items():
+        assert nbytes > 0
+        full = os.path.join(ROOT, path)
+        assert os.path.isfile(full), path
+        assert instance in open(full).read()
