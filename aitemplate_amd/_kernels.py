@@ -87,6 +87,7 @@ EXPORTED_SYMBOLS = [
     "aitamd_attention_set_variant",
     "aitamd_elementwise",
     "aitamd_elementwise_supported",
+    "aitamd_copy_rows",
     "aitamd_gemm_workspace_bytes",
     "aitamd_gemm_rcr_ws",
     "aitamd_gemm_rcr_noalloc",
@@ -166,6 +167,8 @@ def load() -> ctypes.CDLL:
         lib.aitamd_elementwise.argtypes = [i32, i32, vp, vp, vp, i64, i64, ctypes.c_float, i32, vp]
         lib.aitamd_elementwise_supported.restype = i32
         lib.aitamd_elementwise_supported.argtypes = [i32]
+        lib.aitamd_copy_rows.restype = i32
+        lib.aitamd_copy_rows.argtypes = [vp, vp, i64, i64, i64, i64, vp]
         _lib = lib
         return lib
 

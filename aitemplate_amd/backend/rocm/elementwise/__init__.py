@@ -1,1 +1,1 @@
-from . import elementwise  # noqa: F401
+from . import elementwise, strided_copy  # noqa: F401

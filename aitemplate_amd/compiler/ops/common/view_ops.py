@@ -1,5 +1,6 @@
 """View ops: reshape (and flatten via reshape), split and concatenate — ops that move no data on this
-backend.
+backend wherever a GEMM-family op can take the piece as a view, and `strided_copy`, the row copy that the
+strided-view pass puts in their place where none can.
 
 Counterpart of the reshape in python/aitemplate/compiler/ops/common/view_ops.py, reduced
 to static target shapes with at most one -1 (what the GEMM-family graphs use), of
@@ -8,7 +9,7 @@ python/aitemplate/compiler/ops/tensor/concatenate.py:31-170 for the cases that n
 an outer-dim split is a byte offset into its input; a last-dim split or concatenate only
 exists until the strided-view pass has turned it into offsets and row pitches of the GEMM
 ops on either side (the reference's transform_strided_ops.py does the same, and falls back
-to a copy kernel where this backend raises)."""
+to a copy kernel, as the strided-view pass here falls back to `strided_copy`)."""
 from typing import List, Sequence, Union
 
 from ...base import IntImm, IntVar, Operator, Tensor
@@ -102,9 +103,10 @@ class split(_view):
     the split nn.MultiheadAttention applies to the packed [3, batch, heads, seq, head_dim]
     projection.  A split along the last dim makes pieces that are strided views (`strided_view_of`
     = (x, dim, first element)); every consumer has to be an op that can read an operand through an
-    offset and a row pitch, and the strided-view pass of compile_model rewires them to x.  The
-    reference materialises every split with a copy kernel unless a later pass removes it
-    (split.py:172-214)."""
+    offset and a row pitch, and the strided-view pass of compile_model rewires them to x.  Every other
+    piece (a split along a middle dim, a piece that is a graph output or feeds an op that reads contiguous
+    tensors only) becomes a `strided_copy` in that pass.  The reference materialises every split with a
+    copy kernel unless a later pass removes it (split.py:172-214)."""
 
     def __init__(self):
         super().__init__()
@@ -123,9 +125,6 @@ class split(_view):
         if not all(isinstance(d, IntImm) for d in shape[dim:]):
             raise NotImplementedError("split needs static shapes from the split dim on")
         contiguous = all(isinstance(d, IntImm) and d.value() == 1 for d in shape[:dim])
-        if not contiguous and dim != rank - 1:
-            raise NotImplementedError("split along a middle dim would need a copy kernel; only dim 0 (or a dim "
-                                      "behind dims of size 1) and the last dim are supported")
         size = shape[dim].value()
         if isinstance(split_size_or_sections, (list, tuple)):
             sizes = [int(v.value()) if isinstance(v, IntImm) else int(v) for v in split_size_or_sections]
@@ -169,12 +168,13 @@ class split(_view):
 
 
 class concatenate(_view):
-    """torch.cat(tensors, dim) along the last dim, for inputs that GEMM-family ops write.
+    """torch.cat(tensors, dim).
 
-    The op is a placeholder: the strided-view pass of compile_model makes every producer write its
-    columns of the output directly (offset + row pitch of its C accessor) and drops the op.  An
-    input that no such op produces (a graph input, a constant, a tensor with other consumers) would
-    need the reference's copy kernel (backend/rocm/tensor/concatenate.py) and raises there."""
+    The op is a placeholder: the strided-view pass of compile_model makes every GEMM-family producer of a
+    last-dim concatenate write its columns of the output directly (offset + row pitch of its C accessor),
+    gives every other input (a graph input, a constant, a tensor with other consumers, any input of a
+    concatenate along another dim) a `strided_copy` into its rows of the output, as the reference's copy
+    kernel does (backend/rocm/tensor/concatenate.py), and drops the op."""
 
     def __init__(self):
         super().__init__()
@@ -190,9 +190,9 @@ class concatenate(_view):
         if not -rank <= dim < rank:
             raise RuntimeError(f"concatenate dim ({dim}) expected to be less than rank ({rank})")
         dim %= rank
-        if dim != rank - 1:
-            raise NotImplementedError("concatenate along a dim other than the last would need a copy kernel")
         first = inputs[0]._attrs["shape"]
+        if not all(isinstance(d, IntImm) for d in first[dim + 1:]):
+            raise NotImplementedError("concatenate needs static shapes behind the concatenated dim")
         total = 0
         for t in inputs:
             shape = t._attrs["shape"]
@@ -216,3 +216,58 @@ class concatenate(_view):
 
     def _get_op_attributes(self):
         return {}
+
+
+def copy_geometry(func_attrs):
+    """(full tensor, piece tensor, row bytes, pitch bytes of the full tensor, byte offset into it) of a
+    strided_copy op."""
+    src, dst = func_attrs["inputs"][0], func_attrs["outputs"][0]
+    full, piece = (src, dst) if func_attrs["copy_kind"] == "slice" else (dst, src)
+    dim = func_attrs["copy_dim"]
+    inner = get_dtype_size(full.dtype())
+    for d in full._attrs["shape"][dim + 1:]:
+        inner *= d.value()
+    length = piece._attrs["shape"][dim].value()
+    return full, piece, length * inner, full._attrs["shape"][dim].value() * inner, func_attrs["copy_start"] * inner
+
+
+class strided_copy(Operator):
+    """One piece of a split copied out of its input ("slice"), or one input of a concatenate copied into
+    its place in the output ("place"): rows of `length * inner` elements, `full * inner` elements apart on
+    the strided side, where inner is the product of the dims behind `dim`.  Created by the strided-view
+    pass only; one launch of the library's row copy.  Stands for the reference's split and concatenate
+    kernels (python/aitemplate/backend/common/split_common.py, concatenate_common.py)."""
+
+    def __init__(self, kind: str, dim: int, start: int):
+        super().__init__()
+        assert kind in ("slice", "place")
+        self._attrs["op"] = "strided_copy"
+        self._attrs["copy_kind"] = kind
+        self._attrs["copy_dim"] = dim
+        self._attrs["copy_start"] = start
+        self._attrs["has_profiler"] = False
+
+    def bind(self, src: Tensor, dst: Tensor) -> None:
+        """Wire the op between two existing tensors (the pass replaces a view by it)."""
+        full, piece = (src, dst) if self._attrs["copy_kind"] == "slice" else (dst, src)
+        dim = self._attrs["copy_dim"]
+        if not all(isinstance(d, IntImm) for d in full._attrs["shape"][dim:]):
+            raise NotImplementedError("a split or concatenate that needs a copy needs static shapes from its dim on")
+        if len(piece._attrs["shape"]) != len(full._attrs["shape"]):
+            raise RuntimeError("strided_copy: rank mismatch")
+        self._attrs["inputs"] = [src]
+        self._attrs["outputs"] = [dst]
+        self._set_depth()
+        dst._attrs["src_ops"].add(self)
+
+    def geometry(self):
+        return copy_geometry(self._attrs)
+
+    def _get_op_attributes(self):
+        return {"kind": self._attrs["copy_kind"], "dim": self._attrs["copy_dim"], "start": self._attrs["copy_start"]}
+
+    def gen_function(self) -> str:
+        from ....backend import registry
+        from ....backend.target import Target
+
+        return registry.get(f"{Target.current().name()}.strided_copy.gen_function")(self._attrs)

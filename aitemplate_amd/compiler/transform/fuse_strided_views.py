@@ -12,13 +12,14 @@ rewrites that matter for the GEMM family:
   through `output_accessors[0].update_base_tensor(cat_output, dim, first element)`; the
   concatenate leaves the graph and its output has one producer per input.
 
-The reference keeps a split or concatenate it cannot fuse and runs a copy kernel for it.  This
-backend has GEMM-family kernels only, so a piece whose consumer (or producer) cannot take a view
-raises NotImplementedError, naming the tensor and the op.
+The reference keeps a split or concatenate it cannot fuse and runs a copy kernel for it.  Here a piece
+whose consumer (or producer) cannot take a view, and every piece of a split or concatenate along a dim
+other than the last, gets a `strided_copy` op: one launch of the library's row copy per piece.
 """
 from typing import List
 
 from ..base import Operator, Tensor
+from ..ops.common.view_ops import strided_copy
 from .toposort import toposort
 from .transform_utils import get_sorted_ops
 
@@ -59,19 +60,32 @@ def can_write_strided(op: Operator) -> bool:
     return _is_plain_gemm(name) or _is_bmm(name)
 
 
+def _piece_needs_copy(piece: Tensor, outputs: List[Tensor]) -> bool:
+    x, dim, _ = piece._attrs["strided_view_of"]
+    if dim != len(x._attrs["shape"]) - 1:
+        return True  # (accessors describe an offset and a pitch of the last dim only)
+    if piece._attrs["is_output"] or any(piece is o for o in outputs):
+        return True
+    for op in piece.dst_ops():
+        for i, t in enumerate(op._attrs["inputs"]):
+            if t is piece and not can_read_strided(op, i):
+                return True
+    return False
+
+
 def _rewire_split_piece(piece: Tensor, outputs: List[Tensor]) -> None:
     x, dim, start = piece._attrs["strided_view_of"]
-    if piece._attrs["is_output"] or any(piece is o for o in outputs):
-        raise NotImplementedError(
-            f"a piece of a last-dim split ({piece._attrs['name']}) is a graph output: that needs a copy kernel, "
-            "which this backend does not have")
+    if _piece_needs_copy(piece, outputs):
+        # the piece becomes a tensor of its own, filled by a row copy out of x
+        piece._attrs["strided_view_of"] = None
+        piece._attrs["is_view_of"] = None
+        for producer in list(piece.src_ops()):
+            piece._attrs["src_ops"].discard(producer)
+        strided_copy("slice", dim, start).bind(x, piece)
+        return
     for op in list(piece.dst_ops()):
         hit = [i for i, t in enumerate(op._attrs["inputs"]) if t is piece]
         for i in hit:
-            if not can_read_strided(op, i):
-                raise NotImplementedError(
-                    f"op {op._attrs['op']} cannot read input {i} through an offset and a row pitch, which a piece "
-                    "of a last-dim split is; only GEMM-family operands and residuals can")
             op._attrs["input_accessors"][i].update_base_tensor(x, dim, start)
         op._attrs["inputs"] = [x if t is piece else t for t in op._attrs["inputs"]]
         piece._attrs["dst_ops"].discard(op)
@@ -101,33 +115,28 @@ def _fuse_concats(graph: List[Tensor], outputs: List[Tensor]) -> bool:
             continue
         out = cat._attrs["outputs"][0]
         dim = cat._attrs["concat_dim"]
-        seen = set()
+        times = {}
+        for t in cat._attrs["inputs"]:
+            times[id(t)] = times.get(id(t), 0) + 1
         start = 0
         out._attrs["src_ops"].discard(cat)
+        last_dim = dim == len(out._attrs["shape"]) - 1
         for t in cat._attrs["inputs"]:
             producers = list(t.src_ops())
             width = t._attrs["shape"][dim].value()
-            why = None
-            if id(t) in seen:
-                why = "appears twice in the concatenate"
-            elif len(producers) != 1 or not can_write_strided(producers[0]):
-                why = "is not written by a GEMM-family op that can write through an offset and a row pitch"
-            elif t._attrs["is_output"] or any(t is o for o in outputs):
-                why = "is a graph output as well"
-            elif len(list(t.dst_ops())) != 1:
-                why = "has other consumers"
-            elif t._attrs["is_view_of"] is not None:
-                why = "is a view"
-            if why is not None:
-                raise NotImplementedError(
-                    f"concatenate input {t._attrs['name']} {why}: that needs a copy kernel, which this backend "
-                    "does not have")
-            seen.add(id(t))
-            producer = producers[0]
-            producer._attrs["output_accessors"][0].update_base_tensor(out, dim, start)
-            producer._attrs["outputs"] = [out]
-            out._attrs["src_ops"].add(producer)
+            fusable = (last_dim and times[id(t)] == 1 and len(producers) == 1 and can_write_strided(producers[0])
+                       and not (t._attrs["is_output"] or any(t is o for o in outputs))
+                       and len(list(t.dst_ops())) == 1 and t._attrs["is_view_of"] is None)
             t._attrs["dst_ops"].discard(cat)
+            if fusable:
+                producer = producers[0]
+                producer._attrs["output_accessors"][0].update_base_tensor(out, dim, start)
+                producer._attrs["outputs"] = [out]
+                out._attrs["src_ops"].add(producer)
+            else:
+                # a graph input, a constant, a tensor somebody else reads or writes through a view, an input that
+                # appears twice, any input of a concatenate along another dim: copied into its rows of the output
+                strided_copy("place", dim, start).bind(t, out)
             start += width
         changed = True
     return changed

@@ -197,3 +197,63 @@ extern "C" int aitamd_elementwise(int func, int dtype, const void* a, const void
   if (e != hipSuccess) return fail("aitamd_elementwise: launch failed: %s", hipGetErrorString(e));
   return 0;
 }
+
+// ---- strided row copy ----------------------------------------------------------------------------------------
+// The copy a split or a concatenate needs when no GEMM-family op can take the piece as a view: `rows` rows of
+// `row_bytes` bytes from src (rows `src_pitch` bytes apart) to dst (rows `dst_pitch` bytes apart).  Takes the place
+// of the reference's generated split and concatenate kernels (python/aitemplate/backend/common/split_common.py,
+// concatenate_common.py, instantiated by backend/rocm/tensor/split.py and concatenate.py).  Bound: HBM, 2 x
+// rows x row_bytes; 16, 4 or 2 bytes per lane and access, whichever pointers, pitches and row length allow.
+namespace aitamd {
+namespace {
+
+template <class V>
+__global__ void __launch_bounds__(256) copy_rows_kernel(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
+                                                       int64_t rows, int64_t row_units, int64_t src_pitch, int64_t dst_pitch) {
+  // grid.x walks a row in units of V, grid.y (and a stride loop) the rows
+  const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (u >= row_units) return;
+  for (int64_t r = blockIdx.y; r < rows; r += gridDim.y)
+    reinterpret_cast<V*>(dst + r * dst_pitch)[u] = reinterpret_cast<const V*>(src + r * src_pitch)[u];
+}
+
+template <class V>
+hipError_t launch_copy_rows(const void* src, void* dst, int64_t rows, int64_t row_bytes, int64_t src_pitch,
+                            int64_t dst_pitch, hipStream_t stream) {
+  const int64_t units = row_bytes / (int64_t)sizeof(V);
+  const int64_t gx = (units + 255) / 256;
+  const int64_t gy = rows < 65535 ? rows : 65535;
+  hipLaunchKernelGGL(copy_rows_kernel<V>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, stream,
+                     static_cast<const unsigned char*>(src), static_cast<unsigned char*>(dst), rows, units, src_pitch,
+                     dst_pitch);
+  return hipGetLastError();
+}
+
+}  // namespace
+}  // namespace aitamd
+
+extern "C" int aitamd_copy_rows(const void* src, void* dst, int64_t rows, int64_t row_bytes, int64_t src_pitch_bytes,
+                                int64_t dst_pitch_bytes, void* stream) {
+  using namespace aitamd;
+  if (rows < 0 || row_bytes < 0) return fail("aitamd_copy_rows: negative size");
+  if (rows == 0 || row_bytes == 0) return 0;
+  if (!src || !dst) return fail("aitamd_copy_rows: null pointer");
+  if (src_pitch_bytes < row_bytes || dst_pitch_bytes < row_bytes)
+    return fail("aitamd_copy_rows: a row pitch (%lld, %lld) is smaller than the row (%lld bytes)",
+                (long long)src_pitch_bytes, (long long)dst_pitch_bytes, (long long)row_bytes);
+  if ((row_bytes + 255) / 256 > 0x7fffffffll) return fail("aitamd_copy_rows: row too long");
+  const uintptr_t all = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | (uintptr_t)row_bytes |
+      (uintptr_t)src_pitch_bytes | (uintptr_t)dst_pitch_bytes;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  hipError_t e;
+  if ((all & 15) == 0)
+    e = launch_copy_rows<uint4>(src, dst, rows, row_bytes, src_pitch_bytes, dst_pitch_bytes, s);
+  else if ((all & 3) == 0)
+    e = launch_copy_rows<uint32_t>(src, dst, rows, row_bytes, src_pitch_bytes, dst_pitch_bytes, s);
+  else if ((all & 1) == 0)
+    e = launch_copy_rows<uint16_t>(src, dst, rows, row_bytes, src_pitch_bytes, dst_pitch_bytes, s);
+  else
+    e = launch_copy_rows<unsigned char>(src, dst, rows, row_bytes, src_pitch_bytes, dst_pitch_bytes, s);
+  if (e != hipSuccess) return fail("aitamd_copy_rows: launch failed: %s", hipGetErrorString(e));
+  return 0;
+}

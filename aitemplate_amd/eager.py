@@ -10,7 +10,7 @@ a missing library or a CPU tensor raises.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -385,4 +385,59 @@ def elementwise(func: str, a: torch.Tensor, b=None, out: Optional[torch.Tensor] 
     rc = lib.aitamd_elementwise(fid, _TORCH_DTYPE_ID[a.dtype], _p(a), b_ptr, _p(out), a.numel(), b_period, b_value, swap,
                                 _stream_ptr())
     _kernels.check(rc, f"elementwise({func})")
+    return out
+
+
+def split(x: torch.Tensor, sizes, dim: int) -> Tuple[torch.Tensor, ...]:
+    """torch.split(x, sizes, dim) with every piece a new contiguous tensor, one strided row copy per piece
+    (python/aitemplate/compiler/ops/tensor/split.py:31-170)."""
+    lib = _kernels.load()
+    if not x.is_cuda or not x.is_contiguous():
+        raise ValueError("x must be a contiguous GPU tensor")
+    dim %= x.dim()
+    if sum(sizes) != x.shape[dim]:
+        raise ValueError(f"split sizes {list(sizes)} do not add up to {x.shape[dim]}")
+    rows = 1
+    for d in x.shape[:dim]:
+        rows *= d
+    inner = x.element_size()
+    for d in x.shape[dim + 1:]:
+        inner *= d
+    outs, start = [], 0
+    for n in sizes:
+        o = torch.empty(*x.shape[:dim], n, *x.shape[dim + 1:], dtype=x.dtype, device=x.device)
+        rc = lib.aitamd_copy_rows(ctypes.c_void_p(x.data_ptr() + start * inner), _p(o), rows, n * inner, x.shape[dim] * inner, n * inner,
+                                  _stream_ptr())
+        _kernels.check(rc, "split")
+        outs.append(o)
+        start += n
+    return tuple(outs)
+
+
+def concatenate(tensors, dim: int) -> torch.Tensor:
+    """torch.cat(tensors, dim) as one strided row copy per input
+    (python/aitemplate/compiler/ops/tensor/concatenate.py:31-170)."""
+    lib = _kernels.load()
+    first = tensors[0]
+    dim %= first.dim()
+    for t in tensors:
+        if not t.is_cuda or not t.is_contiguous() or t.dtype != first.dtype:
+            raise ValueError("inputs must be contiguous GPU tensors of one dtype")
+        if list(t.shape[:dim]) + list(t.shape[dim + 1:]) != list(first.shape[:dim]) + list(first.shape[dim + 1:]):
+            raise ValueError("inputs differ in a dim other than the concatenated one")
+    total = sum(t.shape[dim] for t in tensors)
+    out = torch.empty(*first.shape[:dim], total, *first.shape[dim + 1:], dtype=first.dtype, device=first.device)
+    rows = 1
+    for d in first.shape[:dim]:
+        rows *= d
+    inner = first.element_size()
+    for d in first.shape[dim + 1:]:
+        inner *= d
+    start = 0
+    for t in tensors:
+        n = t.shape[dim]
+        rc = lib.aitamd_copy_rows(_p(t), ctypes.c_void_p(out.data_ptr() + start * inner), rows, n * inner, n * inner, total * inner,
+                                  _stream_ptr())
+        _kernels.check(rc, "concatenate")
+        start += n
     return out

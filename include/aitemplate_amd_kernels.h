@@ -276,6 +276,15 @@ AITAMD_API int aitamd_elementwise(int func, int dtype, const void* a, const void
 /* 1 when aitamd_elementwise implements FuncEnum value `func` (instance filtering at compile time). */
 AITAMD_API int aitamd_elementwise_supported(int func);
 
+/* Strided row copy: `rows` rows of `row_bytes` bytes from src (rows src_pitch_bytes apart) to dst (rows
+ * dst_pitch_bytes apart); the two ranges must not overlap.  What a split or a concatenate becomes when no GEMM-family
+ * op can take the piece as a view (a piece [..., n_i, inner] of x[..., n, inner] is prod(leading dims) rows of
+ * n_i * inner elements out of rows n * inner elements apart).  Replaces the kernels the reference generates in
+ * python/aitemplate/backend/common/split_common.py:479-530 and concatenate_common.py:661-800 (ROCm entries:
+ * python/aitemplate/backend/rocm/tensor/split.py, concatenate.py). */
+AITAMD_API int aitamd_copy_rows(const void* src, void* dst, int64_t rows, int64_t row_bytes, int64_t src_pitch_bytes,
+                                int64_t dst_pitch_bytes, void* stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -570,8 +570,9 @@ def test_split_is_a_view_with_byte_offsets():
     assert [d.value() for d in b.shape()] == [1, 7, 4] and b._attrs["view_offset_bytes"] == 3 * 4 * 2
     parts = ops.split()(Tensor([10, 4], name="u", is_input=True), 4)  # torch semantics: 4, 4, 2
     assert [p.shape()[0].value() for p in parts] == [4, 4, 2]
-    with pytest.raises(NotImplementedError, match="middle dim"):
-        ops.split()(Tensor([2, 10, 4], name="w", is_input=True), 5, dim=1)
+    # a split along a middle dim makes strided pieces (the strided-view pass gives each a row copy)
+    m0, m1 = ops.split()(Tensor([2, 10, 4], name="w", is_input=True), 5, dim=1)
+    assert m1._attrs["strided_view_of"][1:] == (1, 5) and [d.value() for d in m1.shape()] == [2, 5, 4]
     with pytest.raises(RuntimeError, match="does not match"):
         ops.split()(Tensor([10, 4], name="t", is_input=True), [3, 3], dim=0)
     # offsets accumulate through views of views and reach the generated bindings
@@ -651,40 +652,88 @@ def test_last_dim_split_and_concatenate_become_offsets_and_pitches(tmp_path, mon
         assert f"&m, &{e}_input0_dim_1" in model_src
 
 
-def test_strided_views_that_need_a_copy_kernel_are_refused():
+def _ops_of(graph):
+    from aitemplate_amd.compiler.transform.transform_utils import get_sorted_ops
+
+    return [op for op in get_sorted_ops(graph) if not op._attrs.get("is_view_op")]
+
+
+def test_strided_views_that_no_gemm_can_take_become_row_copies():
+    from aitemplate_amd.compiler.ops.common.view_ops import copy_geometry
+
     N, K = 16, 32
     X = Tensor([8, 2 * K], name="x", is_input=True)
-    W, B = Tensor([N, K], name="w", is_input=True), Tensor([N], name="b", is_input=True)
+    B = Tensor([N], name="b", is_input=True)
+    # a piece read by an op without accessors: a copy of 8 rows of K elements out of rows 2 K apart
     xa, xb = ops.split()(X, K, dim=1)
-    # a piece read by an op without accessors, a piece that is an output
     out = ops.reshape()(xb, [4, -1])
     out._attrs["is_output"] = True
-    with pytest.raises(NotImplementedError, match="cannot read input 0 through an offset"):
-        transform.fuse_strided_views(transform.toposort(out), [out])
+    g = transform.fuse_strided_views(transform.toposort(out), [out])
+    (cp,) = _ops_of(g)
+    assert cp._attrs["op"] == "strided_copy" and cp._attrs["copy_kind"] == "slice"
+    assert cp._attrs["inputs"] == [X] and cp._attrs["outputs"] == [xb]
+    assert xb._attrs["is_view_of"] is None and xb._attrs["strided_view_of"] is None
+    assert copy_geometry(cp._attrs)[2:] == (K * 2, 2 * K * 2, K * 2)
+    # a piece that is a graph output
     xa, xb = ops.split()(X, K, dim=1)
     xa._attrs["is_output"] = True
-    with pytest.raises(NotImplementedError, match="graph output"):
-        transform.fuse_strided_views(transform.toposort(xa), [xa])
+    (cp,) = _ops_of(transform.fuse_strided_views(transform.toposort(xa), [xa]))
+    assert cp._attrs["op"] == "strided_copy" and cp._attrs["copy_start"] == 0 and cp._attrs["outputs"] == [xa]
     # a bias cannot be a view
     b0, b1 = ops.split()(Tensor([1, 2 * N], name="b2", is_input=True), N, dim=1)
     # (dims of size 1 in front: this is the contiguous kind of split, not a strided view)
     assert "strided_view_of" not in b1._attrs
-    # concatenate of a graph input, of a tensor with a second consumer, along another dim
+    # concatenate of a GEMM output and a graph input: the GEMM writes its columns, the input is copied into its
+    Z = Tensor([8, N], name="z", is_input=True)
     y = ops.gemm_rcr_bias()(X, Tensor([N, 2 * K], name="w2", is_input=True), B)
-    cat = ops.concatenate()([y, Tensor([8, N], name="z", is_input=True)], dim=1)
+    cat = ops.concatenate()([y, Z], dim=1)
     cat._attrs["is_output"] = True
-    with pytest.raises(NotImplementedError, match="is not written by a GEMM-family op"):
-        transform.fuse_strided_views(transform.toposort(cat), [cat])
+    kinds = sorted(op._attrs["op"] for op in _ops_of(transform.fuse_strided_views(transform.toposort(cat), [cat])))
+    assert kinds == ["gemm_rcr_bias", "strided_copy"]
+    (cp,) = [op for op in cat.src_ops() if op._attrs["op"] == "strided_copy"]
+    assert cp._attrs["copy_kind"] == "place" and cp._attrs["inputs"] == [Z] and cp._attrs["copy_start"] == N
+    assert copy_geometry(cp._attrs)[2:] == (N * 2, 2 * N * 2, N * 2)
+    # a tensor with a second consumer keeps its own buffer and is copied
     y = ops.gemm_rcr_bias()(X, Tensor([N, 2 * K], name="w3", is_input=True), B)
     y2 = ops.gemm_rcr_bias()(y, Tensor([N, N], name="w4", is_input=True), B)
     cat = ops.concatenate()([y, y2], dim=-1)
     cat._attrs["is_output"] = True
-    with pytest.raises(NotImplementedError, match="has other consumers"):
-        transform.fuse_strided_views(transform.toposort(cat), [cat])
-    with pytest.raises(NotImplementedError, match="other than the last"):
-        ops.concatenate()([y, y2], dim=0)
+    g = transform.fuse_strided_views(transform.toposort(cat), [cat])
+    assert sorted(op._attrs["op"] for op in _ops_of(g)) == ["gemm_rcr_bias", "gemm_rcr_bias", "strided_copy"]
+    assert y._attrs["src_ops"] and [op._attrs["op"] for op in y.src_ops()] == ["gemm_rcr_bias"]
+    # along another dim every input is copied: rows = 1, the whole tensor one row
+    y = ops.gemm_rcr_bias()(X, Tensor([N, 2 * K], name="w5", is_input=True), B)
+    cat = ops.concatenate()([y, Z], dim=0)
+    cat._attrs["is_output"] = True
+    g = transform.fuse_strided_views(transform.toposort(cat), [cat])
+    copies = [op for op in _ops_of(g) if op._attrs["op"] == "strided_copy"]
+    assert len(copies) == 2 and sorted(c._attrs["copy_start"] for c in copies) == [0, 8]
+    assert copy_geometry(copies[0]._attrs)[2:4] == (8 * N * 2, 16 * N * 2)
     with pytest.raises(RuntimeError, match="dim 0 differs"):
         ops.concatenate()([y, Tensor([9, N], name="z2", is_input=True)], dim=1)
+
+
+def test_row_copy_codegen_for_a_middle_dim_split(tmp_path, monkeypatch):
+    """[batch, 10, 4] split along dim 1 into 3 + 7: two generated functions with literal geometry, called with the
+    dynamic batch as the number of rows."""
+    from aitemplate_amd.backend import codegen
+    from aitemplate_amd.compiler.base import IntVar
+    from aitemplate_amd.testing import detect_target
+
+    batch = IntVar([1, 8], name="batch")
+    X = Tensor([batch, 10, 4], name="x", is_input=True)
+    a, b = ops.split()(X, [3, 7], dim=1)
+    a._attrs["name"], a._attrs["is_output"] = "out_a", True
+    b._attrs["name"], b._attrs["is_output"] = "out_b", True
+    with detect_target():
+        g = transform.fuse_strided_views(transform.toposort([a, b]), [a, b])
+        transform.name_graph(g)
+        transform.mark_param_tensor(g, [a, b])
+        pairs = codegen.gen_function_src(g, str(tmp_path), "m")
+    srcs = sorted(open(src).read() for src, _ in pairs)
+    assert len(srcs) == 2
+    assert "aitamd_copy_rows(static_cast<const char*>(src) + 0, dst, rows, 24, 80, 24, stream)" in srcs[0]
+    assert "aitamd_copy_rows(static_cast<const char*>(src) + 24, dst, rows, 56, 80, 56, stream)" in srcs[1]
 
 
 def test_multihead_attention_block_compiles_to_three_kernels(tmp_path, monkeypatch):
