@@ -217,10 +217,30 @@ __global__ void __launch_bounds__(256) copy_rows_kernel(const unsigned char* __r
     reinterpret_cast<V*>(dst + r * dst_pitch)[u] = reinterpret_cast<const V*>(src + r * src_pitch)[u];
 }
 
+// rows shorter than a workgroup: consecutive lanes run on through the rows (one division per lane)
+template <class V>
+__global__ void __launch_bounds__(256) copy_short_rows_kernel(const unsigned char* __restrict__ src,
+                                                             unsigned char* __restrict__ dst, int64_t total_units,
+                                                             uint32_t row_units, int64_t src_pitch, int64_t dst_pitch) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total_units; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / row_units;
+    const int64_t u = i - r * row_units;
+    reinterpret_cast<V*>(dst + r * dst_pitch)[u] = reinterpret_cast<const V*>(src + r * src_pitch)[u];
+  }
+}
+
 template <class V>
 hipError_t launch_copy_rows(const void* src, void* dst, int64_t rows, int64_t row_bytes, int64_t src_pitch,
                             int64_t dst_pitch, hipStream_t stream) {
   const int64_t units = row_bytes / (int64_t)sizeof(V);
+  if (units < 256) {
+    const int64_t total = rows * units;
+    const int64_t blocks = (total + 255) / 256;
+    hipLaunchKernelGGL(copy_short_rows_kernel<V>, dim3((unsigned)(blocks < (1 << 20) ? blocks : (1 << 20))), dim3(256), 0,
+                       stream, static_cast<const unsigned char*>(src), static_cast<unsigned char*>(dst), total,
+                       (uint32_t)units, src_pitch, dst_pitch);
+    return hipGetLastError();
+  }
   const int64_t gx = (units + 255) / 256;
   const int64_t gy = rows < 65535 ? rows : 65535;
   hipLaunchKernelGGL(copy_rows_kernel<V>, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, stream,
