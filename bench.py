@@ -487,17 +487,12 @@ def main():
                    "instance_selected_by": "--algo" if algo_given else args.select},
         "roofline": roofline,
     }
-    # The headline is measured; the legs below add to the line and must not be able to take it away.  The CPU
-    # baseline and the legs of this library come first, the legs that call other libraries last.
+    # The headline is measured; the legs below add to the line and must not be able to take it away.
     def leg(key, fn):
         try:
             line[key] = fn()
         except Exception as e:
             line[key] = {"error": f"{type(e).__name__}: {e}"}
-    if not args.no_cpu_baseline:
-        leg("cpu_baseline", lambda: cpu_baseline(torch))
-    if not args.no_in_abi:
-        leg("in_abi", lambda: in_abi(torch))
     if not args.no_vendor_baseline:
         leg("power_and_vendor_baseline", lambda: power_and_vendor_baseline(torch, eager, case, algo))
     del case
@@ -505,6 +500,10 @@ def main():
         leg("other_configs", lambda: other_configs(torch, eager, _kernels, max(20, min(200, args.steps // 2)),
                                                    max(5, min(50, args.warmup // 2)),
                                                    vendor_baseline=not args.no_vendor_baseline))
+    if not args.no_in_abi:
+        leg("in_abi", lambda: in_abi(torch))
+    if not args.no_cpu_baseline:
+        leg("cpu_baseline", lambda: cpu_baseline(torch))
     print(json.dumps(line))
 
 
