@@ -544,7 +544,6 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
     const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
     // first step: the rest of the slab whose first portion went out in the previous slab's last step
-    // first step: the rest of the slab whose first portion went out in the previous slab's last step
     issue_part(c_P, c_L, d1, kt1, st1);
     if constexpr (ACTIVE) {
       half1_reads(cur_st);
