@@ -12,6 +12,8 @@
 //   aitamd_profiler gemm <op_name> <dtype:0|1> M N K [split_k]
 //   aitamd_profiler bmm  bmm_rcr   <dtype> B M N K
 //   aitamd_profiler attn bmm_softmax_bmm_permute <dtype> B M N K O heads [causal]
+//   aitamd_profiler ew   <FuncEnum value> <dtype> numel [b_period]   (stand-alone element-wise kernel)
+//   aitamd_profiler copy rows <dtype, unused> rows row_bytes pitch_bytes  (row copy out of a pitched buffer)
 // environment: AITAMD_PROF_WARMUP (default 3), AITAMD_PROF_ITERS (default 10),
 //              AITAMD_PROF_ALGO=<name or index> restricts the run to one instance.
 #include <hip/hip_runtime.h>
@@ -336,11 +338,62 @@ int profile_attention(int dtype, int64_t B, int64_t M, int64_t N, int64_t K, int
   return 0;
 }
 
+// Element-wise kernel and row copy: one line each, operands rotating through the same kind of pool.
+int profile_streaming(const std::string& kind, int func, int dtype, int64_t n0, int64_t n1, int64_t n2) {
+  const bool ew = kind == "ew";
+  const int64_t numel = ew ? n0 : 0, b_period = ew ? n1 : 0;
+  const int64_t rows = ew ? 0 : n0, row_bytes = ew ? 0 : n1, pitch = ew ? 0 : n2;
+  if (ew ? numel <= 0 : (rows <= 0 || row_bytes <= 0 || pitch < row_bytes)) {
+    fprintf(stderr, "bad sizes\n");
+    return 2;
+  }
+  const size_t in_bytes = ew ? (size_t)numel * 2 : (size_t)rows * pitch;
+  const size_t out_bytes = ew ? (size_t)numel * 2 : (size_t)rows * row_bytes;
+  int sets = (int)(kPoolTargetBytes / (in_bytes + out_bytes)) + 1;
+  if (sets > kMaxSets) sets = kMaxSets;
+  if (sets < 2) sets = 2;
+  std::vector<DeviceBuf> in(sets), in2(sets), out(sets);
+  for (int s = 0; s < sets; ++s) {
+    in[s] = s == 0 ? alloc_random(in_bytes / 2, dtype, 1.0f, 31) : alloc_copy_of(in[0]);
+    if (ew && b_period > 0) in2[s] = s == 0 ? alloc_random((size_t)b_period, dtype, 1.0f, 32) : alloc_copy_of(in2[0]);
+    out[s].bytes = out_bytes;
+    HIP_OK(hipMalloc(&out[s].p, out_bytes));
+  }
+  const int warmup = env_int("AITAMD_PROF_WARMUP", 3);
+  const int iters = env_int("AITAMD_PROF_ITERS", 10);
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  hipEvent_t e0, e1;
+  HIP_OK(hipEventCreate(&e0));
+  HIP_OK(hipEventCreate(&e1));
+  auto launch = [&](int s) {
+    return ew ? aitamd_elementwise(func, dtype, in[s].p, b_period > 0 ? in2[s].p : nullptr, out[s].p, numel,
+                                   b_period > 0 ? b_period : 1, 0.5f, 0, stream)
+              : aitamd_copy_rows(in[s].p, out[s].p, rows, row_bytes, pitch, row_bytes, stream);
+  };
+  for (int i = 0; i < warmup; ++i) {
+    if (launch(i % sets) != 0) {
+      fprintf(stderr, "launch failed: %s\n", aitamd_last_error());
+      return 3;
+    }
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipEventRecord(e0, stream));
+  for (int i = 0; i < iters; ++i) launch(i % sets);
+  HIP_OK(hipEventRecord(e1, stream));
+  HIP_OK(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  printf("OP:%s,TIME:%.6f,WS:0\n", ew ? "elementwise" : "copy_rows", ms / (iters > 0 ? iters : 1));
+  HIP_OK(hipStreamDestroy(stream));
+  return 0;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
   if (argc < 4) {
-    fprintf(stderr, "usage: %s gemm|gemm_permute|gemm_layout|bmm|bmm_permute|bmm_layout|attn <op> <dtype> dims...\n", argv[0]);
+    fprintf(stderr, "usage: %s gemm|gemm_permute|gemm_layout|bmm|bmm_permute|bmm_layout|attn|ew|copy <op> <dtype> dims...\n", argv[0]);
     return 2;
   }
   const std::string kind = argv[1];
@@ -392,6 +445,14 @@ int main(int argc, char** argv) {
     const bool add = op.size() > 4 && op.compare(op.size() - 4, 4, "_add") == 0;
     if (batched) return profile_gemm_like(add ? "bmm_add" : "bmm_rcr", dtype, d[0], d[1], d[2], d[3], true, perm);
     return profile_gemm_like("bmm_rcr", dtype, 1, d[0], d[1], d[2], true, perm);
+  }
+  if (kind == "ew") {
+    if (d.size() < 1) return 2;
+    return profile_streaming(kind, atoi(op.c_str()), dtype, d[0], d.size() > 1 ? d[1] : 0, 0);
+  }
+  if (kind == "copy") {
+    if (d.size() < 3) return 2;
+    return profile_streaming(kind, 0, dtype, d[0], d[1], d[2]);
   }
   if (kind == "attn") {
     if (d.size() < 6) return 2;
