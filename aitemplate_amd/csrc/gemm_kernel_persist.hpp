@@ -36,7 +36,6 @@ namespace aitamd {
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int MT_ = 32>
 struct GemmTilePersist {
   static constexpr int MT = MT_, KSTEP = MT == 32 ? 16 : 32, QN = 64 / MT, ACC_N = MT * MT / 64;
-  static constexpr int SB = 32;  // rows of an epilogue strip pass (one or two block rows)
   static constexpr int BM = BM_, BN = BN_, BK = BK_;
   static constexpr int WGM = WGM_, WGN = WGN_, NS = NS_;
   static constexpr int NW = WGM * WGN;
@@ -54,13 +53,21 @@ struct GemmTilePersist {
   static constexpr int ROWS_PER_LOAD = 64 / CPR;
   static constexpr int A_LOADS = BM / ROWS_PER_LOAD;
   static constexpr int B_LOADS = BN / ROWS_PER_LOAD;
-  static constexpr int LOADS_PER_STEP = (A_LOADS + B_LOADS) / NW;  // wave-loads per slab per wave
+  // Wave-loads per slab per wave.  L_MAIN consecutive blocks for every wave; where the blocks do not divide over the
+  // waves (320 rows of A: 36 blocks on 8 waves) the last XTRA blocks of A go out as one more load of every wave,
+  // block A_MAIN + wave % XTRA (fetched by NW / XTRA waves each: the same bytes to the same place).
+  static constexpr int L_MAIN = (A_LOADS + B_LOADS) / NW;
+  static constexpr int XTRA = (A_LOADS + B_LOADS) - L_MAIN * NW;
+  static constexpr int A_MAIN = A_LOADS - XTRA;
+  static constexpr int LOADS_PER_STEP = L_MAIN + (XTRA > 0 ? 1 : 0);
   static constexpr int L_P0 = (LOADS_PER_STEP + 1) / 2;            // issued in a slab's last step
   static constexpr int STAGE_ELEMS = (BM + BN) * BK;
   static constexpr int RING_BYTES = NS * STAGE_ELEMS * 2;
   // wave-private epilogue strip: 32 rows x WTN elements of the output type
   static constexpr int STRIP_CHUNKS = WTN / 8;  // 16-byte chunks per strip row
   static constexpr int STRIP_PITCH = WTN * 2;
+  // rows of an epilogue strip pass: 32 (one or two block rows) where the LDS has room for it beside the ring
+  static constexpr int SB = RING_BYTES + NW * 32 * STRIP_PITCH <= 160 * 1024 ? 32 : 16;
   static constexpr int STRIP_BYTES = SB * STRIP_PITCH;
   static constexpr int ROWS_PER_PASS = 64 / STRIP_CHUNKS;
   static constexpr int PASSES = SB / ROWS_PER_PASS;
@@ -69,7 +76,9 @@ struct GemmTilePersist {
   static_assert((MT == 32 && KK == 2) || (MT == 16 && KK == 1 && MI % 2 == 0), "a slab is multiplied in two halves");
   static_assert(WTM % SB == 0, "a wave's rows are whole strip passes");
   static_assert(NS >= 4, "needs one slab in flight behind the one being waited for");
-  static_assert((A_LOADS + B_LOADS) % NW == 0, "slab loads must divide over the waves");
+  static_assert(XTRA == 0 || (XTRA <= A_LOADS && NW % XTRA == 0 && L_P0 < LOADS_PER_STEP - 1),
+                "left-over blocks: all of A, fetched as the last load of the slab's second portion");
+  static_assert(SB % MT == 0, "a strip pass is whole block rows");
   static_assert(STRIP_CHUNKS == 4 || STRIP_CHUNKS == 8 || STRIP_CHUNKS == 16, "strip swizzle needs 2^k chunks");
   static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
 };
@@ -125,19 +134,24 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   // The loads of one portion ([0, L_P0) or [L_P0, L)) share one LDS base: the instruction's immediate offset
   // places the later ones (it shifts the global address as well, which the lane offsets take back).  Writing
   // the LDS base register before every load instead costs a fifth of the whole kernel's time.
-  static_assert(Tile::A_LOADS % L == 0, "a wave's blocks must not straddle A and B");
-  const bool loads_a = wave * L < Tile::A_LOADS;
+  constexpr int LM = Tile::L_MAIN, XTRA = Tile::XTRA;
+  static_assert(Tile::A_MAIN % LM == 0, "a wave's consecutive blocks must not straddle A and B");
+  const bool loads_a = wave * LM < Tile::A_MAIN;
+  // first LDS block of the wave's consecutive loads (A's blocks come first in a stage, its left-over ones last)
+  const int l_block0 = wave * LM + (loads_a ? 0 : XTRA);
+  const int l_block_x = Tile::A_MAIN + (XTRA > 0 ? wave % (XTRA > 0 ? XTRA : 1) : 0);
   const int l_row = lane / Tile::CPR;
   const int l_slot = lane % Tile::CPR;
   uint32_t l_off[L];
   int l_chunk_k[L];
 #pragma unroll
   for (int i = 0; i < L; ++i) {
-    const int j = wave * L + i;
-    const int row = (loads_a ? j : j - Tile::A_LOADS) * Tile::ROWS_PER_LOAD + l_row;
+    const bool extra = XTRA > 0 && i == LM;  // the left-over block of A: always A, placed by its own LDS base
+    const int j = wave * LM + i;
+    const int row = (extra ? l_block_x : (loads_a ? j : j - Tile::A_MAIN)) * Tile::ROWS_PER_LOAD + l_row;
     const int chunk = l_slot ^ ((row / Tile::RPW) % Tile::CPR);
-    const int in_portion = SHORT_K ? 0 : (i < L_P0 ? i : i - L_P0);
-    l_off[i] = (uint32_t)(((int64_t)row * (loads_a ? p.lda : p.ldb) + chunk * 8) * 2 - in_portion * 1024);
+    const int in_portion = (SHORT_K || extra) ? 0 : (i < L_P0 ? i : i - L_P0);
+    l_off[i] = (uint32_t)(((int64_t)row * ((loads_a || extra) ? p.lda : p.ldb) + chunk * 8) * 2 - in_portion * 1024);
     l_chunk_k[i] = chunk * 8;
   }
 
@@ -161,7 +175,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   // Descriptor of the operand panel (A or B) this wave fetches for the workgroup's i-th tile.  Past the last tile
   // the ring keeps turning on a zero-sized buffer: every lane is out of range, nothing is fetched, and the number
   // of loads in flight per step stays constant.
-  auto tile_desc = [&](int i, __amdgpu_buffer_rsrc_t& d) __attribute__((always_inline)) {
+  // (dx: the A panel, for the left-over block every wave fetches; only tiles with such blocks use it)
+  auto tile_desc = [&](int i, __amdgpu_buffer_rsrc_t& d, __amdgpu_buffer_rsrc_t& dx) __attribute__((always_inline)) {
     if (i < my_tiles) {
       const TileCoord c = tile_coord(i);
       const int rows_a = (p.M - c.m0) < c.rows ? (p.M - c.m0) : c.rows;
@@ -172,21 +187,27 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       const uint32_t bytes_a = rows_a > 0 ? clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2) : 0u;
       const uint32_t bytes_b = clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2);
       d = make_rsrc(loads_a ? Ab : Bb, loads_a ? bytes_a : bytes_b);
+      if constexpr (XTRA > 0) dx = make_rsrc(Ab, bytes_a);
     } else {
       d = make_rsrc(p.a, 0);
+      if constexpr (XTRA > 0) dx = d;
     }
   };
 
   // Issue wave-loads [I0, I1) of K-slab `kt` of the tile behind `d` into ring stage `stage`.  No state, no
   // branches: the slab loop calls it between MFMAs and has to stay one basic block for the interleave to hold.
-  auto issue_part = [&](auto i0_c, auto i1_c, const __amdgpu_buffer_rsrc_t& d, int kt, int stage) __attribute__((always_inline)) {
+  auto issue_part = [&](auto i0_c, auto i1_c, const __amdgpu_buffer_rsrc_t& d, const __amdgpu_buffer_rsrc_t& dx, int kt,
+                        int stage) __attribute__((always_inline)) {
     constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
     const int k0 = kt * BK;
-    T* dst = smem + stage * Tile::STAGE_ELEMS + (wave * L + I0) * 512;  // 1 KiB per wave-load
+    T* dst = smem + stage * Tile::STAGE_ELEMS + (l_block0 + I0) * 512;  // 1 KiB per wave-load
     static_for<I0, I1>([&](auto i_c) {
       constexpr int i = decltype(i_c)::value;
       const uint32_t off = (k0 + l_chunk_k[i] < p.K) ? l_off[i] + (uint32_t)(k0 * 2) : kOobOffset;
-      if constexpr (SHORT_K)
+      if constexpr (XTRA > 0 && i == LM)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(dx, (lds_void*)(smem + stage * Tile::STAGE_ELEMS + l_block_x * 512), 16,
+                                                 off, 0, 0, 0);
+      else if constexpr (SHORT_K)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (lds_void*)(dst + (i - I0) * 512), 16, off, 0, 0, 0);
       else
         __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (lds_void*)dst, 16, off, 0, (i - I0) * 1024, 0);
@@ -461,8 +482,9 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   constexpr std::integral_constant<int, L_P0> c_P{};
   constexpr std::integral_constant<int, L> c_L{};
   static_assert(L_P0 > 0 && L_P0 < L, "a slab goes out in two portions");
-  __amdgpu_buffer_rsrc_t rd, nrd;  // this wave's operand panel of the current and of the next tile
-  tile_desc(0, rd);
+  __amdgpu_buffer_rsrc_t rd, nrd;    // this wave's operand panel of the current and of the next tile
+  __amdgpu_buffer_rsrc_t rdx, nrdx;  // and their A panels, for tiles with left-over blocks
+  tile_desc(0, rd, rdx);
   if constexpr (SHORT_K) {
     // Short K: the loader is more than a tile ahead and wraps at places that depend on k_tiles, so it keeps its
     // position as state and tests for the wrap after every slab it has issued (the conditional costs the
@@ -472,16 +494,16 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       if (++ld_kt == k_tiles) {
         ld_kt = 0;
         ++ld_i;
-        tile_desc(ld_i, rd);
+        tile_desc(ld_i, rd, rdx);
       }
     };
 #pragma unroll
     for (int s = 0; s < NS - 2; ++s) {
-      issue_part(c_0, c_P, rd, ld_kt, s);
-      issue_part(c_P, c_L, rd, ld_kt, s);
+      issue_part(c_0, c_P, rd, rdx, ld_kt, s);
+      issue_part(c_P, c_L, rd, rdx, ld_kt, s);
       advance();
     }
-    issue_part(c_0, c_P, rd, ld_kt, NS - 2);
+    issue_part(c_0, c_P, rd, rdx, ld_kt, NS - 2);
     wait_vmcnt<(NS - 3) * L + L_P0>();
     __builtin_amdgcn_s_barrier();
     int rd_stage = 0;
@@ -495,7 +517,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
         const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
         const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
-        issue_part(c_P, c_L, rd, ld_kt, st1);
+        issue_part(c_P, c_L, rd, rdx, ld_kt, st1);
         advance();
         if (active) {
           half1_reads(cur_st);
@@ -506,7 +528,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         }
         wait_vmcnt<(NS - 3) * L>();
         __builtin_amdgcn_s_barrier();
-        issue_part(c_0, c_P, rd, ld_kt, st2);
+        issue_part(c_0, c_P, rd, rdx, ld_kt, st2);
         if (active) {
           half2_reads(nxt_st);
           if (kt == 0)
@@ -525,18 +547,18 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 #pragma unroll
   for (int s = 0; s < NS - 2; ++s) {
     // (portion by portion: the lane offsets assume the immediate offsets of a portion's loads)
-    issue_part(c_0, c_P, rd, s, s);
-    issue_part(c_P, c_L, rd, s, s);
+    issue_part(c_0, c_P, rd, rdx, s, s);
+    issue_part(c_P, c_L, rd, rdx, s, s);
   }
-  issue_part(c_0, c_P, rd, NS - 2, NS - 2);
+  issue_part(c_0, c_P, rd, rdx, NS - 2, NS - 2);
   wait_vmcnt<(NS - 3) * L + L_P0>();
   __builtin_amdgcn_s_barrier();
   int rd_stage = 0;
   load_frags(smem, 0, af[0], bf[0]);
 
   // one K-slab: ACTIVE waves multiply, the others only keep the ring turning
-  auto slab = [&](auto active_c, auto first_c, const __amdgpu_buffer_rsrc_t& d1, int kt1,
-                  const __amdgpu_buffer_rsrc_t& d2, int kt2) __attribute__((always_inline)) {
+  auto slab = [&](auto active_c, auto first_c, const __amdgpu_buffer_rsrc_t& d1, const __amdgpu_buffer_rsrc_t& d1x, int kt1,
+                  const __amdgpu_buffer_rsrc_t& d2, const __amdgpu_buffer_rsrc_t& d2x, int kt2) __attribute__((always_inline)) {
     constexpr bool ACTIVE = decltype(active_c)::value, FIRST = decltype(first_c)::value;
     const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
     const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
@@ -544,7 +566,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     const int st1 = rd_stage + D1 >= NS ? rd_stage + D1 - NS : rd_stage + D1;
     const int st2 = rd_stage + D2 >= NS ? rd_stage + D2 - NS : rd_stage + D2;
     // first step: the rest of the slab whose first portion went out in the previous slab's last step
-    issue_part(c_P, c_L, d1, kt1, st1);
+    issue_part(c_P, c_L, d1, d1x, kt1, st1);
     if constexpr (ACTIVE) {
       half1_reads(cur_st);
       half1_mfmas(first_c);
@@ -555,7 +577,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     // slab, and the next slab's first fragments are fetched under this slab's last MFMAs
     wait_vmcnt<(NS - 3) * L>();
     __builtin_amdgcn_s_barrier();
-    issue_part(c_0, c_P, d2, kt2, st2);
+    issue_part(c_0, c_P, d2, d2x, kt2, st2);
     if constexpr (ACTIVE) {
       half2_reads(nxt_st);
       half2_mfmas(first_c, nxt_st);
@@ -566,20 +588,20 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     rd_stage = nx_stage;
   };
   auto tile_slabs = [&](auto active_c) __attribute__((always_inline)) {
-    slab(active_c, std::true_type{}, rd, D1, rd, D2);
-    for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, std::false_type{}, rd, kt + D1, rd, kt + D2);
+    slab(active_c, std::true_type{}, rd, rdx, D1, rd, rdx, D2);
+    for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, std::false_type{}, rd, rdx, kt + D1, rd, rdx, kt + D2);
 #pragma unroll
     for (int t = 0; t < D2; ++t) {
       if (t == 0)
-        slab(active_c, std::false_type{}, rd, k_tiles - 1, nrd, 0);
+        slab(active_c, std::false_type{}, rd, rdx, k_tiles - 1, nrd, nrdx, 0);
       else
-        slab(active_c, std::false_type{}, nrd, t - 1, nrd, t);
+        slab(active_c, std::false_type{}, nrd, nrdx, t - 1, nrd, nrdx, t);
     }
   };
 
   for (int i = 0; i < my_tiles; ++i) {
     const TileCoord cur = tile_coord(i);
-    tile_desc(i + 1, nrd);
+    tile_desc(i + 1, nrd, nrdx);
     // waves whose rows lie outside a half tile keep the ring turning (their share of the loads, the
     // waits and the barriers) but multiply and store nothing; a half tile is always the last item
     const bool active = wm * Tile::WTM < cur.rows;
@@ -590,6 +612,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       tile_slabs(std::false_type{});
     }
     rd = nrd;
+    if constexpr (XTRA > 0) rdx = nrdx;
   }
   // no LDS-DMA may be in flight into a workgroup that has ended
   wait_vmcnt<0>();
