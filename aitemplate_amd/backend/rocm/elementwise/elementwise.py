@@ -6,6 +6,7 @@ group through backend/common/elementwise_common.py) for the one-op case: an `ele
 absorbed becomes one launch of `aitamd_elementwise`.  The output has the shape of the larger operand; the other
 operand is a constant number or a tensor whose dims, leading 1s dropped, are the output's trailing dims (a bias row,
 a same-shape residual, a one-element tensor): it tiles the flattened output with period prod(its dims)."""
+import math
 from typing import Any, Dict, List
 
 from ....compiler.ops.common.elementwise import standalone_plan
@@ -22,6 +23,17 @@ def _signature(func_name: str) -> str:
             "hipStream_t stream)")
 
 
+def float_literal(value: float) -> str:
+    """C++ spelling of a constant operand: a float literal, or the <cmath> macros for the values that have none
+    (repr() gives 'inf' and 'nan', and 'inff' is not C++)."""
+    value = float(value)
+    if math.isnan(value):
+        return "NAN"
+    if math.isinf(value):
+        return "INFINITY" if value > 0 else "-INFINITY"
+    return f"{value!r}f"
+
+
 def gen_function(func_attrs: Dict[str, Any]) -> str:
     func_name = func_attrs["name"]
     a, b, value, swap = standalone_plan(func_attrs)
@@ -29,7 +41,7 @@ def gen_function(func_attrs: Dict[str, Any]) -> str:
     return f"""{common.HEADER}
 {_signature(func_name)} {{
   check_rc(aitamd_elementwise({func_attrs["func"].value} /* {func_attrs["func"].name} */, {dtype}, a, b, out, numel, b_period,
-                              {value!r}f, {swap}, stream), "{func_name}");
+                              {float_literal(value)}, {swap}, stream), "{func_name}");
 }}
 {common.FOOTER}"""
 

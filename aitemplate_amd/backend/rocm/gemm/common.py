@@ -163,6 +163,7 @@ HEADER = """// generated by aitemplate_amd (ROCm / gfx950 GEMM backend) - do not
 #include <hip/hip_runtime_api.h>
 #include <stdint.h>
 
+#include <cmath>
 #include <stdexcept>
 #include <string>
 

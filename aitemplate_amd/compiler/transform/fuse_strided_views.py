@@ -61,6 +61,7 @@ def can_write_strided(op: Operator) -> bool:
 
 
 def _piece_needs_copy(piece: Tensor, outputs: List[Tensor]) -> bool:
+    """Whatever the other pieces turn out to be, this one cannot be read in place."""
     x, dim, _ = piece._attrs["strided_view_of"]
     if dim != len(x._attrs["shape"]) - 1:
         return True  # (accessors describe an offset and a pitch of the last dim only)
@@ -73,9 +74,46 @@ def _piece_needs_copy(piece: Tensor, outputs: List[Tensor]) -> bool:
     return False
 
 
-def _rewire_split_piece(piece: Tensor, outputs: List[Tensor]) -> None:
+def _residual_pitch(op: Operator, idx: int, copied: dict):
+    """Row pitch the op's residual input `idx` will have once the pass has run: the width of the tensor a piece
+    is read out of when it stays a view, the tensor's own width otherwise."""
+    acc = op._attrs["input_accessors"][idx]
+    if acc.actual_shapes is not None:
+        return acc.row_pitch()
+    t = op._attrs["inputs"][idx]
+    view = t._attrs.get("strided_view_of")
+    if view is not None and id(t) in copied and not copied[id(t)]:
+        return view[0]._attrs["shape"][-1].value()
+    return t._attrs["shape"][-1].value()
+
+
+def _decide_copies(pieces: List[Tensor], outputs: List[Tensor]) -> dict:
+    """id(piece) -> True when the piece becomes a tensor of its own.  The generated launch passes one row pitch for
+    both residuals (`ldd`), so a residual may only be a view when every residual of that op ends up with the same
+    pitch; a piece that fails this is copied, which can change the pitch its partner was checked against, hence
+    the loop (a piece only ever moves from view to copy)."""
+    copied = {id(t): _piece_needs_copy(t, outputs) for t in pieces}
+    changed = True
+    while changed:
+        changed = False
+        for piece in pieces:
+            if copied[id(piece)]:
+                continue
+            for op in piece.dst_ops():
+                inputs = op._attrs["inputs"]
+                res = [i for i in range(3, len(inputs))] if _is_plain_gemm(op._attrs["op"]) else []
+                if len(res) < 2 or not any(inputs[i] is piece for i in res):
+                    continue
+                if len({_residual_pitch(op, i, copied) for i in res}) > 1:
+                    copied[id(piece)] = True
+                    changed = True
+                    break
+    return copied
+
+
+def _rewire_split_piece(piece: Tensor, needs_copy: bool) -> None:
     x, dim, start = piece._attrs["strided_view_of"]
-    if _piece_needs_copy(piece, outputs):
+    if needs_copy:
         # the piece becomes a tensor of its own, filled by a row copy out of x
         piece._attrs["strided_view_of"] = None
         piece._attrs["is_view_of"] = None
@@ -93,19 +131,20 @@ def _rewire_split_piece(piece: Tensor, outputs: List[Tensor]) -> None:
 
 
 def _fuse_splits(graph: List[Tensor], outputs: List[Tensor]) -> bool:
-    changed = False
+    splits = []
     for op in get_sorted_ops(graph):
         if op._attrs["op"] != "split":
             continue
         pieces = [t for t in op._attrs["outputs"] if t._attrs.get("strided_view_of") is not None]
-        if not pieces:
-            continue
+        if pieces:
+            splits.append((op, pieces))
+    copied = _decide_copies([t for _, pieces in splits for t in pieces], outputs)
+    for op, pieces in splits:
         for piece in pieces:
-            _rewire_split_piece(piece, outputs)
+            _rewire_split_piece(piece, copied[id(piece)])
         # nothing reads the pieces any more: the split is unreachable from the outputs
         op._attrs["inputs"][0]._attrs["dst_ops"].discard(op)
-        changed = True
-    return changed
+    return bool(splits)
 
 
 def _fuse_concats(graph: List[Tensor], outputs: List[Tensor]) -> bool:

@@ -153,7 +153,7 @@ namespace {
 
 int attention_entry(const char* who, int dtype, const void* q, const void* k, const void* v, void* out, int64_t B,
                     int64_t M, int64_t N, int64_t K, int64_t O, int64_t G, float scale, int causal,
-                    const int32_t* kv_len, const int32_t* q_len, void* stream) {
+                    const int32_t* kv_len, const int32_t* q_len, bool nan_reset, void* stream) {
   if (dtype != 0 && dtype != 1) return fail("%s: bad dtype %d", who, dtype);
   if (B < 0 || M < 0 || N < 0 || K < 0 || O < 0) return fail("%s: negative dimension", who);
   if (G <= 0 || (B % G) != 0) return fail("%s: batch %lld is not a multiple of heads %lld", who,
@@ -180,6 +180,7 @@ int attention_entry(const char* who, int dtype, const void* q, const void* k, co
   p.causal = causal ? 1 : 0;
   p.kv_len = kv_len;
   p.q_len = q_len;
+  p.nan_reset = nan_reset ? 1 : 0;
   const int ks = (int)((K + 15) / 16) > 0 ? (int)((K + 15) / 16) : 1;
   const int ot = (int)((O + 31) / 32);
   const bool vec = (K % 8 == 0) && (O % 8 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15) == 0) &&
@@ -241,8 +242,10 @@ extern "C" int aitamd_attention_set_variant(int variant) {
 extern "C" int aitamd_bmm_softmax_bmm_permute(int dtype, const void* q, const void* k, const void* v, void* out,
                                               int64_t B, int64_t M, int64_t N, int64_t K, int64_t O, int64_t G,
                                               float scale, int causal, void* stream) {
+  // NaN scores count as -inf: the reference gives this op's kernel ScaleAndResetNaNToMinusInfinity
+  // (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:106, bmm_softmax_bmm.py:99)
   return attention_entry("aitamd_bmm_softmax_bmm_permute", dtype, q, k, v, out, B, M, N, K, O, G, scale, causal, nullptr,
-                         nullptr, stream);
+                         nullptr, true, stream);
 }
 
 extern "C" int aitamd_mem_eff_attention(int dtype, const void* q, const void* k, const void* v, void* out,
@@ -252,6 +255,8 @@ extern "C" int aitamd_mem_eff_attention(int dtype, const void* q, const void* k,
   if (batch < 0 || heads <= 0) return fail("aitamd_mem_eff_attention: bad batch %lld or heads %lld", (long long)batch,
                                            (long long)heads);
   if (batch > 0x7fffffffll / heads) return fail("aitamd_mem_eff_attention: dimension too large");
+  // (a NaN score stays a NaN: the reference's kernel for this op scales only,
+  // python/aitemplate/backend/rocm/attention/mem_eff_attention.py:74)
   return attention_entry("aitamd_mem_eff_attention", dtype, q, k, v, out, batch * heads, seq_q, seq_kv, head_dim,
-                         head_dim_v, heads, scale, causal, lengths_kv, lengths_q, stream);
+                         head_dim_v, heads, scale, causal, lengths_kv, lengths_q, false, stream);
 }

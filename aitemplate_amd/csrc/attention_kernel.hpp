@@ -48,6 +48,8 @@ struct AttnParams {
   // Optional, same form: rows m >= q_len[b / G] of batch entry b are written as zeros, and a workgroup whose rows
   // all lie past that length visits no keys.
   const int32_t* q_len;
+  // Non-zero: a NaN score counts as -inf (its key is left out of the row's softmax) instead of making the row NaN.
+  int32_t nan_reset;
 };
 
 // NW_ waves (32 query rows each) share the K / V tiles; NS_ LDS stages.  The register-staged
@@ -445,8 +447,9 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         const bool need_mask = (nb + 32 * KB > N) || (p.causal && nb + 32 * KB - 1 > m0 + wave_u * 32);
         float alpha = 1.0f;
         vec8 pf[2 * KB];  // P^T fragments of the block's 16-key steps
-        auto softmax_block = [&](auto masked_tag) {
+        auto softmax_block = [&](auto masked_tag, auto nan_tag) {
           constexpr bool MASKED = decltype(masked_tag)::value;
+          constexpr bool NAN_RESET = decltype(nan_tag)::value;  // (implies MASKED)
           bool dead[KB][16];
           if constexpr (MASKED) {
 #pragma unroll
@@ -454,7 +457,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
 #pragma unroll
               for (int e = 0; e < 16; ++e) {
                 const int n = nb + kb * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                dead[kb][e] = (n >= N) || (p.causal && n > q_row);
+                dead[kb][e] = (n >= N) || (p.causal && n > q_row) || (NAN_RESET && s[kb][e] != s[kb][e]);
               }
           }
           float text = -INFINITY;
@@ -491,10 +494,22 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           }
           m_run = m_new;
         };
+        const float m_before = m_run, l_before = l_run;
         if (need_mask)
-          softmax_block(std::true_type{});
+          softmax_block(std::true_type{}, std::false_type{});
         else
-          softmax_block(std::false_type{});
+          softmax_block(std::false_type{}, std::false_type{});
+        // A NaN score (a NaN in Q or in a K row) counts as -inf, i.e. its key is left out, as in the reference, whose
+        // kernel applies ScaleAndResetNaNToMinusInfinity to the scores
+        // (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:106, bmm_softmax_bmm.py:99).  The running
+        // maximum ignores NaNs as it is (fmaxf), and a NaN probability shows in the lane's row sum: the block is redone
+        // with those keys masked.  One compare and one scalar branch per block where there is none.  (mem_eff_attention
+        // runs without the reset: the reference's kernel for it only scales.)
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(l_run != l_run) != 0, 0) && p.nan_reset) {
+          m_run = m_before;
+          l_run = l_before;
+          softmax_block(std::true_type{}, std::true_type{});
+        }
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
           for (int ot = 0; ot < OT; ++ot)

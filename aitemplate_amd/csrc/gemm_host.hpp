@@ -42,6 +42,28 @@ inline int split_k_rule(int64_t tiles, int64_t k_tiles, int cus) {
   return (int)(s < 1 ? 1 : s);
 }
 
+// Compute units of a device, looked up once per device (256 where the device cannot be asked).  The launcher's grid
+// and split-K factor and the instance choice all use this one figure.
+inline int device_cus(int dev) {
+  constexpr int kSlots = 64;
+  static int cus[kSlots] = {};
+  if (dev < 0) dev = 0;
+  int v = cus[dev % kSlots];
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cus[dev % kSlots] = v;
+  }
+  return v;
+}
+inline int current_device_cus() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();  // no device: the instance choice still answers, priced for a 256-CU part
+    return 256;
+  }
+  return device_cus(dev);
+}
+
 // Defined once per (epilogue, dtype) translation unit; nullptr table when that
 // combination is not compiled in.
 GemmAlgoTable gemm_table(int epilogue, int dtype);

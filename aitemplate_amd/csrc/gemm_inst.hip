@@ -92,17 +92,6 @@ struct IsPersistent<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT>> {
   static constexpr bool value = true;
 };
 
-// compute units of a device (looked up once per device)
-inline int device_cus(int dev) {
-  static int cus[kMaxDevices] = {};
-  int v = cus[dev % kMaxDevices];
-  if (v == 0) {
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-    cus[dev % kMaxDevices] = v;
-  }
-  return v;
-}
-
 // Workgroups per tile of a split-K launch: as many as bring the grid up to about one workgroup per CU, each with
 // at least two K-slabs, at most 16; 1 (no splitting, nothing written to the scratch memory) for grids that fill
 // the device anyway.

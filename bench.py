@@ -101,19 +101,34 @@ class PowerSampler:
                 "source": f"{os.path.basename(self.path)} of the card's hwmon, every 20 ms over the last 60 % of the region"}
 
 
-def timed_region(torch, step, steps, warmup, groups=20, graph=False, power=None):
-    """W untimed steps, then exactly K steps between two device synchronisations.  Events on the launch stream
-    bracket the region and cut it into up to `groups` groups of consecutive launches: the region's average and
-    the median of the group averages both come from the same K launches.  With `graph` the K steps are captured
-    once (untimed) and the timed region replays them: for kernels of a few microseconds, whose launches the host
-    cannot issue as fast as the GPU retires them."""
-    for i in range(warmup):
+SETTLE_LAUNCHES = 400      # untimed launches in front of every timed region, whatever --warmup says
+GRAPH_MIN_LAUNCHES = 100   # launches held by the graph a launch-bound configuration is timed with
+
+
+def graph_plan(steps, groups, min_launches=GRAPH_MIN_LAUNCHES):
+    """(launches per captured graph, replays in the timed region).  A graph of one 5 us kernel measures the cost of
+    launching a graph, not the kernel: the graph always holds at least `min_launches` launches, however few steps
+    were asked for, and the timed region replays it once per group."""
+    groups = max(1, min(groups, steps))
+    return max(min_launches, -(-steps // groups)), groups
+
+
+def timed_region(torch, step, steps, warmup, groups=20, graph=False, power=None, settle=SETTLE_LAUNCHES):
+    """`settle` + W untimed steps, then exactly K steps between two device synchronisations.  The settle launches
+    take the region out of the transient after an idle spell (clocks and translation caches need some 30 ms of
+    load; the first 200 launches run up to 1.5x slower), so that the figure does not depend on the W the caller
+    chose.  Events on the launch stream bracket the region and cut it into up to `groups` groups of consecutive
+    launches: the region's average and the median of the group averages both come from the same K launches.  With
+    `graph` the launches are captured once (untimed, graph_plan() says how many) and the timed region replays
+    them: for kernels of a few microseconds, whose launches the host cannot issue as fast as the GPU retires
+    them."""
+    for i in range(settle + warmup):
         step(i)
     torch.cuda.synchronize()
     groups = max(1, min(groups, steps))
     cuts = [steps * g // groups for g in range(groups + 1)]
     if graph:
-        per = steps // groups or 1
+        per, groups = graph_plan(steps, groups)
         g = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()  # default priority
         side.wait_stream(torch.cuda.current_stream())
@@ -122,7 +137,8 @@ def timed_region(torch, step, steps, warmup, groups=20, graph=False, power=None)
                 for i in range(per):
                     step(i)
         torch.cuda.current_stream().wait_stream(side)
-        g.replay()  # untimed: the first replay uploads the graph
+        for _ in range(1 + -(-settle // per)):  # untimed: the first replay uploads the graph
+            g.replay()
         torch.cuda.synchronize()
         cuts = [per * k for k in range(groups + 1)]
         steps = per * groups
@@ -145,7 +161,7 @@ def timed_region(torch, step, steps, warmup, groups=20, graph=False, power=None)
     per_group = [events[k].elapsed_time(events[k + 1]) / (cuts[k + 1] - cuts[k]) for k in range(groups)]
     return {"steps": steps, "wall_ms_per_step": wall_ms / steps,
             "event_ms_per_launch": events[0].elapsed_time(events[-1]) / steps,
-            "median_ms_per_launch": _median(per_group), "groups": groups}
+            "median_ms_per_launch": _median(per_group), "groups": groups, "settle_launches": settle}
 
 
 def _make_pool(torch, op, M, N, K, nres, pool_bytes=600 << 20):
@@ -193,17 +209,21 @@ class GemmCase:
         """A launch lasts a few microseconds: only a replayed graph lets the GPU, not the host, set the pace."""
         return self.flops < 5e9
 
-    def pick_instance(self, iters=15):
+    def pick_instance(self, iters=15, regions=3):
         """Untimed selection pass, the same procedure compile_model's profiling step applies
         (python/aitemplate/compiler/ops/gemm_universal/gemm_common.py:743-829 in the reference):
-        time every instance that supports the problem and keep the fastest."""
-        best, best_ms = -1, float("inf")
-        for algo in self.supported:
-            ms = timed_region(self.torch, self.step_fn(algo), iters * (4 if self.launch_bound else 1), 3, groups=1,
-                              graph=self.launch_bound)["event_ms_per_launch"]
-            if ms < best_ms:
-                best, best_ms = algo, ms
-        return best
+        time every instance that supports the problem and keep the fastest.  Every instance gets `regions`
+        regions, visited round-robin so that a slow spell of the box does not fall on one instance, and counts
+        with its best one."""
+        best_ms = {algo: float("inf") for algo in self.supported}
+        settle = SETTLE_LAUNCHES
+        for _ in range(regions):
+            for algo in self.supported:
+                ms = timed_region(self.torch, self.step_fn(algo), iters * (4 if self.launch_bound else 1), 3, groups=1,
+                                  graph=self.launch_bound, settle=settle)["event_ms_per_launch"]
+                best_ms[algo] = min(best_ms[algo], ms)
+                settle = 0  # the pass itself keeps the device loaded from here on
+        return min(self.supported, key=lambda a: best_ms[a]) if self.supported else -1
 
     def instance_name(self, algo):
         return self.kernels.gemm_algo_names(self.epi, 0)[algo]
@@ -227,7 +247,9 @@ def other_configs(torch, eager, kernels, steps, warmup, vendor_baseline=True):
         r = timed_region(torch, case.step_fn(algo), steps, warmup, graph=graph)
         ws = eager.gemm_workspace_bytes(case.op, algo, case.M, case.N, case.K)
         out[name] = {"op": case.op, "M": case.M, "N": case.N, "K": case.K, "instance": case.instance_name(algo),
-                     "workspace_bytes": ws, "launches": "graph replay" if graph else "direct",
+                     "workspace_bytes": ws,
+                     "launches": f"graph replay, {graph_plan(steps, 20)[0]} launches per graph" if graph else "direct",
+                     "timed_launches": r["steps"], "settle_launches": r["settle_launches"],
                      "ms": round(r["event_ms_per_launch"], 5), "median_ms": round(r["median_ms_per_launch"], 5),
                      "tflops": round(case.flops / r["event_ms_per_launch"] / 1e9, 2),
                      "roofline": _roofline("mfma", case.flops, r["event_ms_per_launch"], r["median_ms_per_launch"])}
@@ -447,6 +469,7 @@ def main():
     roofline["avg_launch_ms"] = round(r["event_ms_per_launch"], 5)
     roofline["median_launch_ms"] = round(r["median_ms_per_launch"], 5)
     roofline["median_of"] = f"{r['groups']} groups of consecutive launches inside the timed region"
+    roofline["settle_launches"] = r["settle_launches"]
     traffic = MEASURED_TRAFFIC.get(instance)
     roofline["traffic"] = traffic[0] if traffic else None
     roofline["traffic_source"] = (f"{traffic[1]} (instance {instance})" if traffic else

@@ -140,7 +140,10 @@ AITAMD_API int aitamd_gemm_rcr_ws(int epilogue, int dtype, int algo,
  * counterpart in the reference (whose ops draw their workspace from the model's allocation).  An instance named by
  * `algo` that needs more than aitamd_gemm_noalloc_scratch_bytes() for this problem is refused with a message;
  * algo = -1 chooses among the instances that fit.  All calls on one GPU share that GPU's array: calls that overlap
- * in time on one GPU (different streams) race - serialise them, or use aitamd_gemm_rcr_ws with separate buffers. */
+ * in time on one GPU (different streams) race - serialise them, or use aitamd_gemm_rcr_ws with separate buffers.
+ * The first call on a GPU looks the array's address up (hipGetSymbolAddress, under a lock).  Under stream capture
+ * that look-up must already have happened: call aitamd_gemm_noalloc_scratch_bytes() once per GPU at set-up, with
+ * that GPU current - it returns the capacity and does the look-up - or make one call outside the capture first. */
 AITAMD_API int aitamd_gemm_rcr_noalloc(int epilogue, int dtype, int algo,
                                        const void* a, const void* b, const void* bias,
                                        const void* d0, const void* d1, void* c,

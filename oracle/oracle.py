@@ -287,13 +287,18 @@ def torch_bmm_rcr_permute(q, k, d1: int) -> torch.Tensor:
 
 def torch_bmm_softmax_bmm_permute(q, k, v, scale: float, num_heads: int, causal: bool = False,
                                   chunk: int = 4) -> torch.Tensor:
-    """softmax(Q K^T * scale) V, output [B/G, M, G, O]; chunked over the batch to bound memory."""
+    """softmax(Q K^T * scale) V, output [B/G, M, G, O]; chunked over the batch to bound memory.  A NaN score
+    counts as -inf (its key is left out): the reference's kernel takes ScaleAndResetNaNToMinusInfinity as the
+    functor between the first product and the softmax
+    (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:106, bmm_softmax_bmm.py:99).  A row whose
+    scores are all NaN is left to PyTorch's softmax here (NaN) and is pinned by nothing."""
     q, k, v = _f(q), _f(k), _f(v)
     B, M, _ = q.shape
     N, O = v.shape[1], v.shape[2]
     out = torch.empty(B, M, O, dtype=torch.float32)
     for s in range(0, B, chunk):
         att = torch.bmm(q[s:s + chunk], k[s:s + chunk].transpose(1, 2)) * scale
+        att = torch.where(torch.isnan(att), torch.full_like(att, float("-inf")), att)
         if causal:
             mask = torch.ones(M, N, dtype=torch.bool).tril()
             att = att.masked_fill(~mask, float("-inf"))

@@ -202,26 +202,31 @@ def test_config_c5_full_size():
     torch.testing.assert_close(got.cpu().float(), want, atol=TOL, rtol=TOL)
 
 
-def test_nan_in_a_key_gives_nan_for_its_batch_entry_only():
-    """A NaN score stays a NaN here, as in PyTorch's softmax (the oracle): every query of the batch entry that
-    holds the bad key row comes out NaN, the other batch entries are untouched.  Composable Kernel, which the
-    reference calls, resets NaN scores to -inf before the softmax instead
-    (python/aitemplate/utils/mk_ck_lib/gemm_operation.py:415-424 instantiates that kernel); that reset is not
-    replicated, and this test pins the difference."""
+def test_nan_in_a_key_leaves_that_key_out():
+    """A NaN score counts as -inf, as in the reference, whose kernel takes ScaleAndResetNaNToMinusInfinity between the
+    first product and the softmax (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:106): every query of
+    the batch entry that holds the bad key row comes out finite and equal to attention without that key; a NaN in a
+    query row resets all of that row's scores, which the reference leaves as 0 / 0 and nothing pins (finite or NaN
+    is accepted there); a NaN in V reaches the output as a NaN."""
     B, M, N, K, O, G = 4, 96, 200, 64, 64, 2
     print(f"case attention NaN key B={B} M={M} N={N} K={K}", flush=True)
     q, k, v = _rand((B, M, K), torch.float16, 11), _rand((B, N, K), torch.float16, 12), _rand((B, N, O), torch.float16, 13)
     k[1, 77, 5] = float("nan")
+    k[1, 199, 0] = float("nan")   # in the masked tail tile as well
+    q[2, 40, 3] = float("nan")
+    v[3, 10, 7] = float("nan")
     want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, K ** -0.5, G, False).half().float()   # [B/G, M, G, O]
     got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
-    assert torch.isnan(want[0, :, 1, :]).all(), "the oracle (PyTorch softmax) propagates the NaN"
-    assert torch.isnan(got[0, :, 1, :]).all()
-    keep = torch.ones(B // G, G, dtype=torch.bool)
-    keep[0, 1] = False
-    for bo in range(B // G):
-        for g in range(G):
-            if keep[bo, g]:
-                torch.testing.assert_close(got[bo, :, g, :], want[bo, :, g, :], atol=TOL, rtol=TOL)
+    assert not torch.isnan(want[0, :, 1, :]).any(), "the oracle resets NaN scores"
+    assert not torch.isnan(got[0, :, 1, :]).any()
+    keep = [n for n in range(N) if n not in (77, 199)]
+    without = oracle.torch_bmm_softmax_bmm_permute(q[1:2], k[1:2, keep], v[1:2, keep], K ** -0.5, 1, False)
+    torch.testing.assert_close(got[0, :, 1, :], without[0, :, 0, :].half().float(), atol=TOL, rtol=TOL)
+    open_rows = torch.zeros(B // G, M, G, dtype=torch.bool)
+    open_rows[1, 40, 0] = True   # the query row whose scores are all NaN
+    assert torch.isnan(got[1, :, 1, 7]).all() and torch.isnan(want[1, :, 1, 7]).all()
+    sel = ~open_rows[..., None].expand_as(got)
+    torch.testing.assert_close(got[sel], want[sel], atol=TOL, rtol=TOL, equal_nan=True)
 
 
 # ---- head dims that leave padding columns in the LDS tiles (K = 16 KS - 8: 24, 40, 56, 88, 120, 152; O = 32 OT - 24)
@@ -272,16 +277,17 @@ def test_large_small_and_all_negative_logits():
 
 
 def test_nan_key_and_lengths_at_head_dim_40(attn_variant):
-    """NaN propagation and the length masks at head dim 40 (padded to 48 / 64 inside LDS), every variant."""
-    B, M, N, K, O, G = 4, 96, 200, 40, 40, 2
+    """The NaN reset and the length masks at head dim 40 (padded to 48 / 64 inside LDS), every variant."""
+    B, M, N, K, O, G = 4, 96, 700, 40, 40, 2
     q, k, v = _rand((B, M, K), torch.float16, 41), _rand((B, N, K), torch.float16, 42), _rand((B, N, O), torch.float16, 43)
     k[1, 77, 5] = float("nan")
+    k[1, 650, 1] = float("nan")
     want = oracle.torch_bmm_softmax_bmm_permute(q, k, v, K ** -0.5, G, False).half().float()
-    got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
-    assert torch.isnan(got[0, :, 1, :]).all() and torch.isnan(want[0, :, 1, :]).all()
-    for bo, g in ((0, 0), (1, 0), (1, 1)):
-        torch.testing.assert_close(got[bo, :, g, :], want[bo, :, g, :], atol=TOL, rtol=TOL)
+    assert not torch.isnan(want).any()
     for mode in (-1, 0, 1, 2, 3):
         attn_variant(mode)
+        print(f"case attention NaN reset head dim 40 variant {mode}", flush=True)
+        got = eager.bmm_softmax_bmm_permute(q.cuda(), k.cuda(), v.cuda(), (G,), scale=K ** -0.5).cpu().float()
+        torch.testing.assert_close(got, want, atol=TOL, rtol=TOL)
         _check_mem_eff(3, 4, 150, 333, 40, 40, [333, 1, 200], causal=False)
         _check_mem_eff(3, 4, 150, 150, 40, 40, [150, 0, 77], causal=True, lens_q=[150, 10, 0])

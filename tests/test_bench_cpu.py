@@ -52,3 +52,50 @@ def test_traffic_table_names_files_that_exist():
         full = os.path.join(ROOT, path)
         assert os.path.isfile(full), path
         assert instance in open(full).read()
+
+
+def test_graph_of_a_launch_bound_configuration_never_holds_fewer_than_100_launches():
+    # the driver's "--steps 20 --warmup 5" reaches other_configs as 20 steps in 20 groups
+    assert bench.graph_plan(20, 20) == (100, 20)
+    assert bench.graph_plan(1, 20) == (100, 1)
+    assert bench.graph_plan(200, 20) == (100, 20)
+    # more steps than 100 per group: the graph grows, the number of replays stays the number of groups
+    assert bench.graph_plan(4000, 20) == (200, 20)
+    assert bench.graph_plan(4001, 20) == (201, 20)
+    assert bench.graph_plan(60, 1) == (100, 1)
+
+
+class _FakeTorch:
+    """Just enough of torch.cuda for timed_region's direct-launch path: events count the steps issued so far."""
+
+    class cuda:
+        issued = 0
+
+        @staticmethod
+        def synchronize():
+            pass
+
+        class Event:
+            def __init__(self, enable_timing=True):
+                self.at = None
+
+            def record(self):
+                self.at = _FakeTorch.cuda.issued
+
+            def elapsed_time(self, other):
+                return float(other.at - self.at)
+
+
+def test_timed_region_runs_settle_and_warmup_untimed_and_times_exactly_k_steps():
+    calls = []
+
+    def step(i):
+        _FakeTorch.cuda.issued += 1
+        calls.append(i)
+
+    _FakeTorch.cuda.issued = 0
+    r = bench.timed_region(_FakeTorch, step, 20, 5, settle=300)
+    assert len(calls) == 300 + 5 + 20
+    assert r["steps"] == 20 and r["settle_launches"] == 300 and r["groups"] == 20
+    assert r["event_ms_per_launch"] == 1.0 and r["median_ms_per_launch"] == 1.0  # one "ms" per fake launch
+    assert bench.SETTLE_LAUNCHES >= 300

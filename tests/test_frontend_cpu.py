@@ -713,6 +713,70 @@ def test_strided_views_that_no_gemm_can_take_become_row_copies():
         ops.concatenate()([y, Tensor([9, N], name="z2", is_input=True)], dim=1)
 
 
+def test_two_residuals_are_views_only_when_they_share_one_row_pitch(tmp_path, monkeypatch):
+    """The generated launch has one `ldd` for both residuals: a piece of a last-dim split may be read in place as a
+    residual only when the op's other residual ends up with the same row pitch; otherwise it is copied, as the
+    reference does for every split it cannot fuse."""
+    M, N, K = 8, 16, 32
+
+    def graph(d0_of, d1_of):
+        X = Tensor([M, K], name="x", is_input=True)
+        W = Tensor([N, K], name="w", is_input=True)
+        B = Tensor([N], name="b", is_input=True)
+        y = ops.gemm_rcr_bias_add_add()(X, W, B, d0_of(), d1_of())
+        y._attrs["name"], y._attrs["is_output"] = "y", True
+        return y
+
+    def piece_of(name, width, index=1):
+        def make():
+            return ops.split()(Tensor([M, width], name=name, is_input=True), N, dim=1)[index]
+        return make
+
+    def plain(name):
+        return lambda: Tensor([M, N], name=name, is_input=True)
+
+    def run(y):
+        g = transform.fuse_strided_views(transform.toposort(y), [y])
+        kinds = sorted(op._attrs["op"] for op in _ops_of(g))
+        (gemm,) = [op for op in _ops_of(g) if op._attrs["op"] == "gemm_rcr_bias_add_add"]
+        return kinds, [gemm._attrs["input_accessors"][i].row_pitch() for i in (3, 4)]
+
+    # a piece and a plain tensor: pitches 2N and N, so the piece is copied
+    kinds, pitches = run(graph(piece_of("r", 2 * N), plain("p")))
+    assert kinds == ["gemm_rcr_bias_add_add", "strided_copy"] and pitches == [N, N]
+    kinds, pitches = run(graph(plain("p"), piece_of("r", 2 * N)))
+    assert kinds == ["gemm_rcr_bias_add_add", "strided_copy"] and pitches == [N, N]
+    # pieces of splits of different widths: both copied
+    kinds, pitches = run(graph(piece_of("r", 2 * N), piece_of("q", 3 * N)))
+    assert kinds == ["gemm_rcr_bias_add_add", "strided_copy", "strided_copy"] and pitches == [N, N]
+    # pieces of splits of the same width (or of one split): both stay views
+    kinds, pitches = run(graph(piece_of("r", 2 * N), piece_of("q", 2 * N, index=0)))
+    assert kinds == ["gemm_rcr_bias_add_add"] and pitches == [2 * N, 2 * N]
+    # the partner has to be copied for a reason of its own (it is a graph output too): then so is the piece
+    X = Tensor([M, K], name="x", is_input=True)
+    q0, q1 = ops.split()(Tensor([M, 2 * N], name="q", is_input=True), N, dim=1)
+    r1 = ops.split()(Tensor([M, 2 * N], name="r", is_input=True), N, dim=1)[1]
+    y = ops.gemm_rcr_bias_add_add()(X, Tensor([N, K], name="w", is_input=True), Tensor([N], name="b", is_input=True), r1, q1)
+    y._attrs["name"], y._attrs["is_output"] = "y", True
+    q1._attrs["is_output"] = True
+    g = transform.fuse_strided_views(transform.toposort([y, q1]), [y, q1])
+    assert sorted(op._attrs["op"] for op in _ops_of(g)) == ["gemm_rcr_bias_add_add", "strided_copy", "strided_copy"]
+
+    # the mixed case compiles (it raised NotImplementedError in the code generator before)
+    monkeypatch.setenv("CI_FLAG", "CIRCLECI")
+    reset_name_counters()
+    y = graph(piece_of("r", 2 * N), plain("p"))
+    import torch
+
+    if torch.cuda.is_available():
+        compile_model(y, detect_target(), str(tmp_path), "mixed_residuals").close()
+    else:
+        with pytest.raises(RuntimeError, match="AITemplateModelContainerCreate"):
+            compile_model(y, detect_target(), str(tmp_path), "mixed_residuals")
+    assert f"const int64_t ldd = N;" in "".join(
+        f.read_text() for f in (tmp_path / "mixed_residuals").glob("gemm_rcr_bias_add_add*.cpp"))
+
+
 def test_row_copy_codegen_for_a_middle_dim_split(tmp_path, monkeypatch):
     """[batch, 10, 4] split along dim 1 into 3 + 7: two generated functions with literal geometry, called with the
     dynamic batch as the number of rows."""
@@ -1034,3 +1098,27 @@ def test_leftover_elementwise_ops_become_standalone_launches(tmp_path, monkeypat
             .standalone_plan()
     with pytest.raises(NotImplementedError, match="with 2 operands is not supported"):
         list(ops.elementwise(ops.FuncEnum.RELU)(h, h).src_ops())[0].standalone_plan()
+
+
+def test_non_finite_constant_operands_are_spelled_as_cmath_macros(tmp_path):
+    """A clamp against float('inf') is a legal graph; repr() would give the literal `inff`."""
+    import subprocess
+
+    from aitemplate_amd.backend.rocm.elementwise.elementwise import float_literal, gen_function
+
+    assert float_literal(2.0) == "2.0f" and float_literal(-0.5) == "-0.5f" and float_literal(1e-8) == "1e-08f"
+    assert float_literal(float("inf")) == "INFINITY" and float_literal(float("-inf")) == "-INFINITY"
+    assert float_literal(float("nan")) == "NAN"
+    X = Tensor([4, 8], name="x", is_input=True)
+    y = ops.elementwise(ops.FuncEnum.MIN)(X, float("inf"))
+    attrs = list(y.src_ops())[0]._attrs
+    attrs["name"] = "elementwise_inf"
+    src = gen_function(attrs)
+    assert "INFINITY, 0, stream" in src and "inff" not in src and "#include <cmath>" in src
+    # the generated function is valid C++ (syntax only: the kernel library's header is the one it includes)
+    f = tmp_path / "ew.cpp"
+    f.write_text(src)
+    r = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+                        f"-I{os.path.join(ROOT, 'include')}", f"-I{os.path.join(ROOT, 'aitemplate_amd', 'static', 'include')}",
+                        str(f)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]

@@ -109,3 +109,73 @@ def test_splitk_without_workspace_runs_unsplit():
     assert eager.gemm_workspace_bytes(op, 0, M, N, K) == 0
     out = eager.gemm(op, x.cuda(), w.cuda(), b.cuda(), algo=0, workspace=eager.new_workspace(64))
     torch.testing.assert_close(out.cpu().float(), want, atol=1e-2, rtol=1e-2)
+
+
+def test_splitk_results_do_not_change_under_cache_pressure():
+    """The workgroups of a tile run on different XCDs, whose L2s are not coherent with each other: the partial tiles
+    are exchanged with write-through stores and a counter.  About 2000 launches over six shapes; before every launch
+    the partial-tile slots of the scratch memory (not its counters) are filled with NaN and a 64 MiB copy goes
+    through the L2s, so a workgroup that read a stale or not yet written slot would show.  Every result is compared
+    bit for bit with the shape's first one (itself checked against the oracle); the test stops at the first batch
+    of launches that holds a mismatch."""
+    op = "gemm_rcr_bias"
+    shapes = [(256, 1024, 1024), (100, 200, 4096), (512, 768, 3072), (64, 256, 8192), (1, 6912, 8320), (192, 320, 2048)]
+    src = torch.empty(64 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    launches_per_shape, batch = 340, 20
+    for M, N, K in shapes:
+        x, w, b, _ = _inputs(M, N, K, 0, torch.float16, seed=M + N + K + 1)
+        want = oracle.torch_gemm(op, x, w, b).half().float()
+        xs, ws, bs = x.cuda(), w.cuda(), b.cuda()
+        best = None
+        for algo, name in _splitk_algos(op):
+            need = eager.gemm_workspace_bytes(op, algo, M, N, K)
+            if need > 4096 and not name.endswith("_k2_splitk") and (best is None or need > best[2]):
+                best = (algo, name, need)
+        assert best is not None, f"no split-K instance splits M={M} N={N} K={K}"
+        algo, name, need = best
+        scratch = eager.new_workspace(need)
+        print(f"case split-K soak {name} M={M} N={N} K={K} workspace={need}", flush=True)
+        first = eager.gemm(op, xs, ws, bs, algo=algo, workspace=scratch)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(first.cpu().float(), want, atol=1e-2, rtol=1e-2)
+        out = torch.empty_like(first)
+        bad = torch.zeros((), dtype=torch.int64, device="cuda")
+        slots = scratch[4096:].view(torch.float32)  # the fp32 partial tiles behind the counters
+        for i in range(launches_per_shape):
+            slots.fill_(float("nan"))
+            dst.copy_(src)
+            eager.gemm(op, xs, ws, bs, out=out, algo=algo, workspace=scratch)
+            bad += (out != first).sum() + torch.isnan(out).sum()
+            if (i + 1) % batch == 0:
+                assert int(bad) == 0, f"{name} M={M} N={N} K={K}: mismatch within launches {i + 1 - batch}..{i}"
+        assert int(bad) == 0
+        assert int(scratch[:4096].to(torch.int32).sum()) == 0
+
+
+def test_splitk_on_two_streams_with_separate_scratch_buffers():
+    """Launches that overlap in time need scratch buffers of their own (the header says so): two streams, each with
+    its own buffer and output, 100 launches each on different shapes, every result equal to a serial run's."""
+    op = "gemm_rcr_bias"
+    cases = []
+    for M, N, K in ((256, 1024, 1024), (64, 256, 8192)):
+        x, w, b, _ = _inputs(M, N, K, 0, torch.float16, seed=M + K)
+        algo, name = [(i, n) for i, n in _splitk_algos(op) if "64x64x64" in n and not n.endswith("_k2_splitk")][0]
+        need = eager.gemm_workspace_bytes(op, algo, M, N, K)
+        assert need > 4096
+        xs, ws, bs = x.cuda(), w.cuda(), b.cuda()
+        serial = eager.gemm(op, xs, ws, bs, algo=algo, workspace=eager.new_workspace(need))
+        torch.cuda.synchronize()
+        torch.testing.assert_close(serial.cpu().float(), oracle.torch_gemm(op, x, w, b).half().float(), atol=1e-2, rtol=1e-2)
+        cases.append((xs, ws, bs, algo, eager.new_workspace(need), serial, torch.cuda.Stream(),  # default priority
+                      torch.zeros((), dtype=torch.int64, device="cuda")))
+    torch.cuda.synchronize()
+    print("case split-K two streams", flush=True)
+    for i in range(100):
+        for xs, ws, bs, algo, scratch, serial, stream, bad in cases:
+            with torch.cuda.stream(stream):
+                out = eager.gemm(op, xs, ws, bs, algo=algo, workspace=scratch)
+                bad += (out != serial).sum()
+    torch.cuda.synchronize()
+    for case in cases:
+        assert int(case[-1]) == 0

@@ -363,3 +363,88 @@ def test_bmm_layouts_brute_force(layout):
                 assert abs(got[bi, m, n].item() - acc) < 1e-4
     if layout == "rcr":
         assert torch.equal(got, oracle.torch_bmm_rcr(a, b))
+
+
+def test_attention_nan_scores_count_as_minus_infinity():
+    """A NaN score leaves its key out of the row's softmax (the reference's ScaleAndResetNaNToMinusInfinity functor,
+    python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:106): against a loop that says `isnan -> -inf`
+    explicitly, and against plain attention over the keys that are left."""
+    B, M, N, K, O, G = 4, 5, 9, 3, 6, 2
+    q, k, v = _rand((B, M, K), seed=1), _rand((B, N, K), seed=2), _rand((B, N, O), seed=3)
+    k[1, 4, 2] = float("nan")      # one key of batch entry 1 is bad for every query
+    q[2, 3, 0] = float("nan")      # one query row of batch entry 2 is bad for every key
+    scale = 0.37
+    want = torch.zeros(B // G, M, G, O, dtype=torch.float64)
+    for b in range(B):
+        for m in range(M):
+            s = []
+            for n in range(N):
+                t = sum(float(q[b, m, kk]) * float(k[b, n, kk]) for kk in range(K)) * scale
+                s.append(-math.inf if math.isnan(t) else t)
+            mx = max(s)
+            if mx == -math.inf:
+                want[b // G, m, b % G, :] = float("nan")  # every score reset: 0 / 0, pinned by nothing
+                continue
+            e = [math.exp(t - mx) for t in s]
+            for o in range(O):
+                want[b // G, m, b % G, o] = sum(e[n] * float(v[b, n, o]) for n in range(N)) / sum(e)
+    got_t = oracle.torch_bmm_softmax_bmm_permute(q, k, v, scale, G).double()
+    got_c = oracle.c_bmm_softmax_bmm_permute(q, k, v, scale, G).double()
+    live = ~torch.isnan(want)
+    assert not live[1, 3, 0].any() and live.sum() == want.numel() - O  # only the all-NaN query row is left open
+    assert torch.allclose(got_t[live], want[live], atol=1e-5)
+    assert torch.allclose(got_c[live], want[live], atol=2e-3, rtol=2e-3)
+    # the same as attention without the bad key
+    keep = [n for n in range(N) if n != 4]
+    ref = oracle.torch_bmm_softmax_bmm_permute(q[1:2], k[1:2, keep], v[1:2, keep], scale, 1).double()
+    assert torch.allclose(got_t[0, :, 1, :], ref[0, :, 0, :], atol=1e-6)
+    # a NaN in V is not a score: it reaches the output of every query of its batch entry
+    v2 = v.clone()
+    v2[0, 2, 1] = float("nan")
+    out = oracle.torch_bmm_softmax_bmm_permute(q, k, v2, scale, G)
+    assert torch.isnan(out[0, :, 0, 1]).all() and not torch.isnan(out[0, :, 0, 0]).any()
+
+
+def test_elementwise_nan_conventions_and_function_table():
+    """torch_elementwise against the reference's device functions written out by hand: MAX / MIN return NaN when
+    either operand is NaN (fmaxf_nan / fminf_nan, backend/rocm/elementwise/custom_math.h:282-310), RELU is
+    `a > 0 ? a : 0`, which sends NaN to 0 (custom_math.h:117), LRELU is `a > 0 ? a : a * slope`."""
+    nan, inf = float("nan"), float("inf")
+    a = torch.tensor([1.0, nan, -2.0, nan, 0.5, -inf, 3.0])
+    b = torch.tensor([nan, 2.0, -3.0, nan, 0.5, 1.0, -inf])
+
+    def by_hand(f):
+        return [f(float(x), float(y)) for x, y in zip(a, b)]
+
+    def same(got, want):
+        want = torch.tensor(want, dtype=torch.float32)
+        return bool((torch.isnan(got) == torch.isnan(want)).all()) and \
+            bool(torch.equal(torch.nan_to_num(got, nan=0.0), torch.nan_to_num(want, nan=0.0)))
+
+    assert same(oracle.torch_elementwise("MAX", a, b),
+                by_hand(lambda x, y: nan if (math.isnan(x) or math.isnan(y)) else max(x, y)))
+    assert same(oracle.torch_elementwise("MIN", a, b),
+                by_hand(lambda x, y: nan if (math.isnan(x) or math.isnan(y)) else min(x, y)))
+    assert same(oracle.torch_elementwise("RELU", a), [x if x > 0 else 0.0 for x in a.tolist()])
+    assert oracle.torch_elementwise("RELU", torch.tensor([nan])).item() == 0.0
+    assert same(oracle.torch_elementwise("LRELU", a, 0.1),
+                [float(torch.tensor(x if x > 0 else x * 0.1, dtype=torch.float32)) for x in a.tolist()])
+    # the rest of the table against the math library on a few points, constants as the second operand included
+    x = torch.tensor([0.25, 1.5, 2.0])
+    y = torch.tensor([2.0, 0.5, 3.0])
+    for name, f in (("ADD", lambda p, q: p + q), ("SUB", lambda p, q: p - q), ("MUL", lambda p, q: p * q),
+                    ("DIV", lambda p, q: p / q), ("POW", lambda p, q: p ** q)):
+        want = torch.tensor([f(float(p), float(q)) for p, q in zip(x, y)])
+        assert torch.allclose(oracle.torch_elementwise(name, x, y), want, rtol=1e-6), name
+        assert torch.allclose(oracle.torch_elementwise(name, x, 2.0),
+                              torch.tensor([f(float(p), 2.0) for p in x]), rtol=1e-6), name
+    for name, f in (("TANH", math.tanh), ("ABS", abs), ("EXP", math.exp), ("SQRT", math.sqrt),
+                    ("SIGMOID", lambda t: 1 / (1 + math.exp(-t))), ("SILU", lambda t: t / (1 + math.exp(-t))),
+                    ("GELU", lambda t: 0.5 * t * (1 + math.erf(t / math.sqrt(2)))),
+                    ("FASTGELU", lambda t: 0.5 * t * (1 + math.tanh(0.7978845608 * (t + 0.044715 * t ** 3)))),
+                    ("COS", math.cos), ("SIN", math.sin), ("SIGN", lambda t: (t > 0) - (t < 0)), ("LOGE", math.log),
+                    ("LOG1P", math.log1p), ("SOFTSIGN", lambda t: t / (1 + abs(t))), ("FLOOR", math.floor),
+                    ("RECIPROCAL", lambda t: 1 / t)):
+        pts = torch.tensor([-1.25, 0.25, 1.5]) if name not in ("SQRT", "LOGE", "LOG1P") else x
+        want = torch.tensor([float(f(float(t))) for t in pts])
+        assert torch.allclose(oracle.torch_elementwise(name, pts), want, rtol=2e-6, atol=1e-7), name

@@ -90,3 +90,51 @@ def test_noalloc_entry_refuses_what_does_not_fit():
     assert "scratch memory" in _kernels.last_error()
     torch.cuda.synchronize()
     assert not bool(out.any()), "a refused call must not launch anything"
+
+
+def test_noalloc_entry_under_stream_capture_and_graph_replay():
+    """Two split-K launches captured into one graph (kernel nodes only; the kernels leave their counters zero, so
+    nothing clears memory between them) and replayed three times with eager work and synchronisations in between:
+    every replay equals the workspace entry's result.  The array's address is looked up beforehand by
+    aitamd_gemm_noalloc_scratch_bytes(); the first call of the no-alloc entry itself happens under capture."""
+    lib = _kernels.load()
+    algo, name = _splitk_algo(lib, "64x64x64")
+    assert lib.aitamd_gemm_noalloc_scratch_bytes() >= (16 << 20)  # (also resolves the array's address)
+    shapes = ((200, 512, 2048), (64, 256, 4096))
+    ops, refs, outs = [], [], []
+    for M, N, K in shapes:
+        x, w, b = (t.cuda() for t in _operands(M, N, K, seed=M + N))
+        need = lib.aitamd_gemm_workspace_bytes(EPI_BIAS, 0, algo, 1, M, N, K)
+        assert need > 0
+        scratch = torch.zeros(need, dtype=torch.uint8, device="cuda")
+        ref = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.aitamd_gemm_rcr_ws(EPI_BIAS, 0, algo, _ptr(x), _ptr(w), _ptr(b), None, None, _ptr(ref), M, N, K, K, K, N, N,
+                                    _ptr(scratch), need, stream)
+        _kernels.check(rc, "aitamd_gemm_rcr_ws")
+        ops.append((x, w, b, M, N, K))
+        refs.append(ref)
+        outs.append(torch.zeros(M, N, dtype=torch.float16, device="cuda"))
+    torch.cuda.synchronize()
+    print(f"case noalloc graph capture {name} shapes {shapes}", flush=True)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()  # default priority
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            handle = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for (x, w, b, M, N, K), out in zip(ops, outs):
+                rc = lib.aitamd_gemm_rcr_noalloc(EPI_BIAS, 0, algo, _ptr(x), _ptr(w), _ptr(b), None, None, _ptr(out),
+                                                 M, N, K, K, K, N, N, handle)
+                _kernels.check(rc, "aitamd_gemm_rcr_noalloc under capture")
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert not any(bool(o.any()) for o in outs), "capture must not run anything"
+    for replay in range(3):
+        for o in outs:
+            o.fill_(float("nan"))  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, ref in zip(outs, refs):
+            assert torch.equal(o, ref), f"replay {replay} differs from the workspace entry"
