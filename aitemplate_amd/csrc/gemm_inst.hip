@@ -52,11 +52,11 @@ struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>, P
       gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>, Epi, PERM, LAYOUT>;
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int NS, int MT, bool PERM, int LAYOUT>
-struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT>, PERM, LAYOUT> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, int MT, int LBM, bool PERM, int LAYOUT>
+struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>, PERM, LAYOUT> {
   // (LAYOUT 4 is not an operand layout: it names the instantiation for tiles of fewer K-slabs than ring stages)
   static constexpr auto value =
-      gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS, MT>, Epi, PERM, LAYOUT == kShortK>;
+      gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>, Epi, PERM, LAYOUT == kShortK>;
 };
 // bit L set: the tile has a kernel for layout L (bit 0, rcr, always)
 template <class Tile>
@@ -87,8 +87,8 @@ template <class Tile>
 struct IsPersistent {
   static constexpr bool value = false;
 };
-template <int BM, int BN, int BK, int WM, int WN, int NS, int MT>
-struct IsPersistent<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT>> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, int MT, int LBM>
+struct IsPersistent<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>> {
   static constexpr bool value = true;
 };
 
@@ -231,11 +231,11 @@ const GemmAlgo kAlgos[] = {
                   GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>::kLdsBytes),                      \
    1, LayoutMask<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>::value,                            \
    &launch_tile<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX>>, nullptr},
-#define AITAMD_GEMM_TILE_PERSIST(BM, BN, BK, WM, WN, NS, MT)                                              \
+#define AITAMD_GEMM_TILE_PERSIST(BM, BN, BK, WM, WN, NS, MT, LBM)                                         \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_persist" #NS "_m" #MT,                \
-   BM, BN, BK, GemmTilePersist<BM, BN, BK, WM, WN, NS, MT>::NT, 8,                                          \
-   GemmTilePersist<BM, BN, BK, WM, WN, NS, MT>::kLdsBytes,                                                  \
-   1, 2, 1, &launch_tile<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT>>, nullptr},
+   BM, BN, BK, GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>::NT, 8,                                     \
+   GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>::kLdsBytes,                                             \
+   1, 2, 1, &launch_tile<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>>, nullptr},
 #define AITAMD_GEMM_TILE_DMA_SPLITK(BM, BN, BK, WM, WN, NS, OCC, PIPE, MT)                                   \
   {"gemm_rcr_" AITAMD_DT_NAME "_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_dma" #NS "_o" #OCC "_p" #PIPE "_m" #MT \
    "_splitk",                                                                                             \

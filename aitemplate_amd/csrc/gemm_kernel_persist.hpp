@@ -33,8 +33,12 @@ namespace aitamd {
 // v_mfma_f32_16x16x32, one K-step per slab, whose blocks are multiplied in two halves (upper and lower block rows)
 // around the slab's barrier; the 16x16x32 form moves half the accumulator registers per multiply-add and sustains
 // 13 % more under the board's power limit on random operands (1.93 against 1.71 PFLOP/s in a loop of MFMAs alone).
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int MT_ = 32>
+// LBM_: rows of the A slab a ring stage holds.  A tile of BM rows whose 16-row blocks do not divide over the waves
+// (224 rows: 14 blocks) takes the next size that does (256: rows past BM are cut off by the panel's buffer
+// descriptor - zero fill, nothing fetched - and no wave reads them).
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int MT_ = 32, int LBM_ = BM_>
 struct GemmTilePersist {
+  static constexpr int LBM = LBM_;
   static constexpr int MT = MT_, KSTEP = MT == 32 ? 16 : 32, QN = 64 / MT, ACC_N = MT * MT / 64;
   static constexpr int BM = BM_, BN = BN_, BK = BK_;
   static constexpr int WGM = WGM_, WGN = WGN_, NS = NS_;
@@ -51,7 +55,7 @@ struct GemmTilePersist {
   static constexpr int RPW32 = (256 / (BK * 2)) > 0 ? (256 / (BK * 2)) : 1;
   static constexpr int RPW = (MT == 16 && RPW32 > 1) ? RPW32 / 2 : RPW32;
   static constexpr int ROWS_PER_LOAD = 64 / CPR;
-  static constexpr int A_LOADS = BM / ROWS_PER_LOAD;
+  static constexpr int A_LOADS = LBM / ROWS_PER_LOAD;
   static constexpr int B_LOADS = BN / ROWS_PER_LOAD;
   // Wave-loads per slab per wave.  L_MAIN consecutive blocks for every wave; where the blocks do not divide over the
   // waves (320 rows of A: 36 blocks on 8 waves) the last XTRA blocks of A go out as one more load of every wave,
@@ -61,19 +65,21 @@ struct GemmTilePersist {
   static constexpr int A_MAIN = A_LOADS - XTRA;
   static constexpr int LOADS_PER_STEP = L_MAIN + (XTRA > 0 ? 1 : 0);
   static constexpr int L_P0 = (LOADS_PER_STEP + 1) / 2;            // issued in a slab's last step
-  static constexpr int STAGE_ELEMS = (BM + BN) * BK;
+  static constexpr int STAGE_ELEMS = (LBM + BN) * BK;
   static constexpr int RING_BYTES = NS * STAGE_ELEMS * 2;
   // wave-private epilogue strip: 32 rows x WTN elements of the output type
   static constexpr int STRIP_CHUNKS = WTN / 8;  // 16-byte chunks per strip row
   static constexpr int STRIP_PITCH = WTN * 2;
   // rows of an epilogue strip pass: 32 (one or two block rows) where the LDS has room for it beside the ring
-  static constexpr int SB = RING_BYTES + NW * 32 * STRIP_PITCH <= 160 * 1024 ? 32 : 16;
+  // (and where a wave's rows are whole 32-row passes)
+  static constexpr int SB = (RING_BYTES + NW * 32 * STRIP_PITCH <= 160 * 1024 && WTM % 32 == 0) ? 32 : 16;
   static constexpr int STRIP_BYTES = SB * STRIP_PITCH;
   static constexpr int ROWS_PER_PASS = 64 / STRIP_CHUNKS;
   static constexpr int PASSES = SB / ROWS_PER_PASS;
   static constexpr int kLdsBytes = RING_BYTES + NW * STRIP_BYTES;
   static_assert(MT == 32 || MT == 16, "MFMA block is 32x32 or 16x16");
-  static_assert((MT == 32 && KK == 2) || (MT == 16 && KK == 1 && MI % 2 == 0), "a slab is multiplied in two halves");
+  static_assert((MT == 32 && KK == 2) || (MT == 16 && KK == 1 && MI >= 2), "a slab is multiplied in two halves");
+  static_assert(LBM >= BM && LBM % ROWS_PER_LOAD == 0, "the A slab in LDS holds the tile's rows");
   static_assert(WTM % SB == 0, "a wave's rows are whole strip passes");
   static_assert(NS >= 4, "needs one slab in flight behind the one being waited for");
   static_assert(XTRA == 0 || (XTRA <= A_LOADS && NW % XTRA == 0 && L_P0 < LOADS_PER_STEP - 1),
@@ -92,7 +98,10 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   using acc_t = typename Mfma::acc_t;
   constexpr int BM = Tile::BM, BN = Tile::BN, BK = Tile::BK, NS = Tile::NS;
   constexpr int MI = Tile::MI, NI = Tile::NI, MT = Tile::MT, KK = Tile::KK, QN = Tile::QN, SB = Tile::SB;
-  constexpr int MH = KK == 1 ? MI / 2 : MI;  // block rows multiplied per half of a slab
+  // block rows multiplied in the first / second half of a slab (one-step slabs: the upper rows, then the lower
+  // ones, one fewer where their number is odd; two-step slabs: all rows in both)
+  constexpr int MH = KK == 1 ? (MI + 1) / 2 : MI;
+  constexpr int MH2 = KK == 1 ? MI - MH : MI;
   constexpr int L = Tile::LOADS_PER_STEP, L_P0 = Tile::L_P0;
   constexpr int SC = Tile::STRIP_CHUNKS;
   typedef __attribute__((address_space(3))) void lds_void;
@@ -219,14 +228,15 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     a_rd[kk] = dma_lds_chunk_elem<Tile>(wm * Tile::WTM + fr, kk * QN + fq);
-    b_rd[kk] = BM * BK + dma_lds_chunk_elem<Tile>(wn * Tile::WTN + fr, kk * QN + fq);
+    b_rd[kk] = Tile::LBM * BK + dma_lds_chunk_elem<Tile>(wn * Tile::WTN + fr, kk * QN + fq);
   }
   // KK == 2: half `hh` of a slab is K-step hh over all block rows (af[hh][0 .. MI), bf[hh][0 .. NI)).
   // KK == 1: half `hh` is block rows hh * MH ... of the one K-step (af[hh][0 .. MH)); both halves use bf[0].
   auto load_a = [&](const T* st, int hh, vec8* af) __attribute__((always_inline)) {
 #pragma unroll
     for (int mi = 0; mi < MH; ++mi)
-      af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[KK == 1 ? 0 : hh] + ((KK == 1 ? hh * MH : 0) + mi) * MT * BK);
+      if (mi < (hh == 0 ? MH : MH2))
+        af[mi] = *reinterpret_cast<const vec8*>(st + a_rd[KK == 1 ? 0 : hh] + ((KK == 1 ? hh * MH : 0) + mi) * MT * BK);
   };
   auto load_b1 = [&](const T* st, int hh, int ni) __attribute__((always_inline)) {
     return *reinterpret_cast<const vec8*>(st + b_rd[KK == 1 ? 0 : hh] + ni * MT * BK);
@@ -277,8 +287,11 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     else
       load_a(nxt_st, 0, af[0]);
   };
-  auto half2_mfmas = [&](auto first_c, const T* nxt_st) __attribute__((always_inline)) {
+  // (FETCH = false: the next slab's fragments are not fetched - a tile's last slab, where they would have to live
+  // through the epilogue; see kRefetch)
+  auto half2_mfmas = [&](auto first_c, const T* nxt_st, auto fetch_c) __attribute__((always_inline)) {
     constexpr bool FIRST = decltype(first_c)::value;
+    constexpr bool FETCH = decltype(fetch_c)::value;
     if constexpr (KK == 2) {
       mfmas(af[1], bf[1]);
     } else {
@@ -286,9 +299,9 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
-        for (int mi = 0; mi < MH; ++mi)
+        for (int mi = 0; mi < MH2; ++mi)
           acc[MH + mi][ni] = Mfma::run(bf[0][ni], af[1][mi], FIRST ? zero : acc[MH + mi][ni]);
-        bf[0][ni] = load_b1(nxt_st, 0, ni);
+        if constexpr (FETCH) bf[0][ni] = load_b1(nxt_st, 0, ni);
       }
     }
   };
@@ -377,26 +390,34 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      vec8 raw[Tile::PASSES], d0v[Tile::PASSES], d1v[Tile::PASSES];
+      // passes in flight at once: all of a strip's, or half of them with two residual operands (three 16-byte
+      // values per pass and lane: all four passes of a 32-row strip at once spilled registers)
+      constexpr int PG = (Epi::kNumD >= 2 && Tile::PASSES >= 4) ? Tile::PASSES / 2 : Tile::PASSES;
 #pragma unroll
-      for (int ps = 0; ps < Tile::PASSES; ++ps) {
-        const int row = ps * Tile::ROWS_PER_PASS + r_row;
-        raw[ps] = *reinterpret_cast<const vec8*>(strip + row * Tile::STRIP_PITCH + ((r_c ^ (row & (SC - 1))) << 4));
-        const uint32_t step_d = (uint32_t)((sb * SB + ps * Tile::ROWS_PER_PASS) * (int)p.ldd * 2);
-        if constexpr (Epi::kNumD >= 1) d0v[ps] = __builtin_bit_cast(vec8, buffer_load_16B(rd0, off_d0 + step_d));
-        if constexpr (Epi::kNumD >= 2) d1v[ps] = __builtin_bit_cast(vec8, buffer_load_16B(rd1, off_d0 + step_d));
-      }
+      for (int p0 = 0; p0 < Tile::PASSES; p0 += PG) {
+        vec8 raw[PG], d0v[PG], d1v[PG];
 #pragma unroll
-      for (int ps = 0; ps < Tile::PASSES; ++ps) {
-        vec8 o;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          // conversion and bias add as one instruction where the type has one; -0.0 is the bias that adds nothing
-          const float xb = Epi::kHasBias ? Tr::to_float_plus(raw[ps][j], one, bf8[j]) : Tr::to_float(raw[ps][j]);
-          o[j] = Tr::from_float(apply_folded<Epi, T>(xb, d0v[ps][j], d1v[ps][j], one));
+        for (int q = 0; q < PG; ++q) {
+          const int ps = p0 + q;
+          const int row = ps * Tile::ROWS_PER_PASS + r_row;
+          raw[q] = *reinterpret_cast<const vec8*>(strip + row * Tile::STRIP_PITCH + ((r_c ^ (row & (SC - 1))) << 4));
+          const uint32_t step_d = (uint32_t)((sb * SB + ps * Tile::ROWS_PER_PASS) * (int)p.ldd * 2);
+          if constexpr (Epi::kNumD >= 1) d0v[q] = __builtin_bit_cast(vec8, buffer_load_16B(rd0, off_d0 + step_d));
+          if constexpr (Epi::kNumD >= 2) d1v[q] = __builtin_bit_cast(vec8, buffer_load_16B(rd1, off_d0 + step_d));
         }
-        const uint32_t off = off_c0 + (uint32_t)((sb * SB + ps * Tile::ROWS_PER_PASS) * (int)p.ldc * 2);
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, NT_BITS);
+#pragma unroll
+        for (int q = 0; q < PG; ++q) {
+          const int ps = p0 + q;
+          vec8 o;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            // conversion and bias add as one instruction where the type has one; -0.0 is the bias that adds nothing
+            const float xb = Epi::kHasBias ? Tr::to_float_plus(raw[q][j], one, bf8[j]) : Tr::to_float(raw[q][j]);
+            o[j] = Tr::from_float(apply_folded<Epi, T>(xb, d0v[q][j], d1v[q][j], one));
+          }
+          const uint32_t off = off_c0 + (uint32_t)((sb * SB + ps * Tile::ROWS_PER_PASS) * (int)p.ldc * 2);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), rc, off, 0, NT_BITS);
+        }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -532,9 +553,9 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         if (active) {
           half2_reads(nxt_st);
           if (kt == 0)
-            half2_mfmas(std::true_type{}, nxt_st);
+            half2_mfmas(std::true_type{}, nxt_st, std::true_type{});
           else
-            half2_mfmas(std::false_type{}, nxt_st);
+            half2_mfmas(std::false_type{}, nxt_st, std::true_type{});
         }
         rd_stage = nx_stage;
       }
@@ -557,9 +578,15 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   load_frags(smem, 0, af[0], bf[0]);
 
   // one K-slab: ACTIVE waves multiply, the others only keep the ring turning
+  // Tiles of more than 128 accumulator registers per lane: the first fragments of the next tile are not held in
+  // registers through the epilogue (36 registers of a 10 x 4 block part, which the epilogue then spills around)
+  // but fetched behind it; the slab they come from has landed and stays in its ring stage.
+  constexpr bool kRefetch = KK == 1 && MI * NI * Tile::ACC_N > 128;
   auto slab = [&](auto active_c, auto first_c, const __amdgpu_buffer_rsrc_t& d1, const __amdgpu_buffer_rsrc_t& d1x, int kt1,
-                  const __amdgpu_buffer_rsrc_t& d2, const __amdgpu_buffer_rsrc_t& d2x, int kt2) __attribute__((always_inline)) {
+                  const __amdgpu_buffer_rsrc_t& d2, const __amdgpu_buffer_rsrc_t& d2x, int kt2,
+                  auto last_c) __attribute__((always_inline)) {
     constexpr bool ACTIVE = decltype(active_c)::value, FIRST = decltype(first_c)::value;
+    constexpr bool FETCH = !(decltype(last_c)::value && kRefetch);
     const T* cur_st = smem + rd_stage * Tile::STAGE_ELEMS;
     const int nx_stage = rd_stage + 1 == NS ? 0 : rd_stage + 1;
     const T* nxt_st = smem + nx_stage * Tile::STAGE_ELEMS;
@@ -579,8 +606,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     __builtin_amdgcn_s_barrier();
     issue_part(c_0, c_P, d2, d2x, kt2, st2);
     if constexpr (ACTIVE) {
-      half2_reads(nxt_st);
-      half2_mfmas(first_c, nxt_st);
+      if constexpr (FETCH) half2_reads(nxt_st);
+      half2_mfmas(first_c, nxt_st, std::integral_constant<bool, FETCH>{});
       // (one-step slabs take no scheduling hints: reads in pairs behind the first MFMAs and loads spread over
       // the rest, the order the hints give two-step slabs, ran 3 to 5 % slower there than the compiler's own)
       if constexpr (KK == 2) sched_step<MI * NI, MI + NI, L_P0>();
@@ -588,15 +615,15 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     rd_stage = nx_stage;
   };
   auto tile_slabs = [&](auto active_c) __attribute__((always_inline)) {
-    slab(active_c, std::true_type{}, rd, rdx, D1, rd, rdx, D2);
-    for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, std::false_type{}, rd, rdx, kt + D1, rd, rdx, kt + D2);
-#pragma unroll
-    for (int t = 0; t < D2; ++t) {
-      if (t == 0)
-        slab(active_c, std::false_type{}, rd, rdx, k_tiles - 1, nrd, nrdx, 0);
-      else
-        slab(active_c, std::false_type{}, nrd, nrdx, t - 1, nrd, nrdx, t);
-    }
+    constexpr std::false_type no{};
+    slab(active_c, std::true_type{}, rd, rdx, D1, rd, rdx, D2, no);
+    for (int kt = 1; kt < k_tiles - D2; ++kt) slab(active_c, no, rd, rdx, kt + D1, rd, rdx, kt + D2, no);
+    slab(active_c, no, rd, rdx, k_tiles - 1, nrd, nrdx, 0, no);
+    static_for<1, D2 - 1>([&](auto t_c) {
+      constexpr int t = decltype(t_c)::value;
+      slab(active_c, no, nrd, nrdx, t - 1, nrd, nrdx, t, no);
+    });
+    slab(active_c, no, nrd, nrdx, D2 - 2, nrd, nrdx, D2 - 1, std::true_type{});
   };
 
   for (int i = 0; i < my_tiles; ++i) {
@@ -608,6 +635,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     if (active) {
       tile_slabs(std::true_type{});
       epilogue(cur);
+      if constexpr (kRefetch) load_frags(smem + rd_stage * Tile::STAGE_ELEMS, 0, af[0], bf[0]);
     } else {
       tile_slabs(std::false_type{});
     }

@@ -417,6 +417,9 @@ def main():
                          "pass over all instances (what compile_model does) or the library's heuristic")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a 256 MiB device copy 5 times (counter calibration for profiler runs)")
+    ap.add_argument("--workload", choices=tuple(SHAPES), default="c2a",
+                    help="diagnostic, for profiler runs of one kernel: time this configuration in the headline "
+                         "region instead of configs[1] (the line then says so in `data` and is not the metric)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--constant-operands", action="store_true",
                     help="diagnostic: time the headline kernel on x = 1, w = 1/K instead of the random operands")
@@ -443,8 +446,11 @@ def main():
         sys.exit(2)
     _kernels.load()
 
-    case = GemmCase(torch, eager, _kernels, "c2a")
+    case = GemmCase(torch, eager, _kernels, args.workload)
     M, N, K = case.M, case.N, case.K
+    diagnostic = args.workload != "c2a"
+    if diagnostic:  # one kernel under a profiler: none of the legs that belong to the metric's line
+        args.no_vendor_baseline = args.no_other_configs = args.no_in_abi = args.no_cpu_baseline = True
     if args.algo.lstrip("-").isdigit():
         algo = int(args.algo)
     else:
@@ -462,7 +468,7 @@ def main():
         # diagnostic run (engine clock on idle multiplier inputs, for the counter profiles): not the metric
         case.pool = [(torch.ones_like(x), torch.full_like(w, 1.0 / K), torch.zeros_like(b), d, out)
                      for (x, w, b, d, out) in case.pool]
-    r = timed_region(torch, case.step_fn(algo), args.steps, args.warmup)
+    r = timed_region(torch, case.step_fn(algo), args.steps, args.warmup, graph=diagnostic and case.launch_bound)
     tflops = case.flops / (r["wall_ms_per_step"] * 1e-3) / 1e12
     instance = case.instance_name(algo)
     roofline = _roofline("mfma", case.flops, r["event_ms_per_launch"], r["median_ms_per_launch"])
@@ -502,7 +508,9 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
-        "data": "constant operands (diagnostic run, not the metric)" if args.constant_operands else "synthetic",
+        "data": ("constant operands (diagnostic run, not the metric)" if args.constant_operands else
+                 f"synthetic; DIAGNOSTIC run of configuration {args.workload} ({case.op} M={M} N={N} K={K}), not the metric"
+                 if diagnostic else "synthetic"),
         "pct_of_fp16_mfma_peak": round(100.0 * tflops / PEAK_FP16_TFLOPS, 2),
         "config": {"workload": "configs[1]: gemm_rcr_bias_gelu fp16 X[24576,768] W[3072,768] bias[3072], "
                                "fp32 accumulate, tanh-GELU fused, inputs resident in HBM, rotating operand sets",
