@@ -166,4 +166,19 @@ AITAMD_DEVICE void map_tile(int wg, int tiles_m, int tiles_n, int batch, int& b,
   tn = in_group / gm;
 }
 
+// Block form of the mapping for one batch whose tile grid divides over the XCDs as xcd_cols column blocks times
+// 8 / xcd_cols row blocks: XCD x works through its own block row by row, so the B panels of the block's few
+// columns are fetched into its L2 once and stay there for every row (the tiles that need an A panel are adjacent
+// in the walk and run at the same time).  Same workgroup -> XCD deal as above: wg % 8 is the XCD.
+AITAMD_DEVICE void map_tile_block(int wg, int tiles_m, int tiles_n, int xcd_cols, int& tm, int& tn) {
+  const int xcd = wg % kNumXcd;
+  const int local = wg / kNumXcd;
+  const int cols = tiles_n / xcd_cols;
+  const int rows = tiles_m / (kNumXcd / xcd_cols);
+  const int cb = xcd % xcd_cols, rb = xcd / xcd_cols;
+  const int r = local / cols;
+  tm = rb * rows + r;
+  tn = cb * cols + (local - r * cols);
+}
+
 }  // namespace aitamd

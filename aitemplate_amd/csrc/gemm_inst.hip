@@ -113,6 +113,25 @@ int64_t workspace_of(const GemmParams& p) {
   return 0;
 }
 
+// Column blocks of the per-XCD block mapping of the persistent kernels (GemmParams::xcd_cols; 0: the grouped
+// mapping).  The grid of one batch is cut into xcd_cols column blocks times 8 / xcd_cols row blocks, one per XCD,
+// where it divides so and the B panels of a block's columns take at most 2.5 MiB; the fewest column blocks that fit
+// are taken, which share an A panel among the most tiles.  An XCD then reads few B panels over and over and every
+// A panel once.  Measured on M=24576 N=3072 K=768 (two column blocks of six tile columns): 158 MB fetched per launch
+// against 176 MB with the grouped mapping, 0.5 % (normally distributed operands) to 2 % (constant ones) less time.
+// The B panels do not stay in the 4 MiB L2 from one block row to the next all the same: a round of 32 tiles streams
+// 4.4 MB of distinct panel data between two uses of a B line (loading A with the non-temporal policy to protect B
+// loses the sharing of A among the tiles of a row: 0.159 against 0.123 ms).
+inline int xcd_column_blocks(const GemmParams& p, int bn, int grid) {
+  if (p.batch != 1 || grid % 8 != 0 || p.tiles_m <= 0 || p.tiles_n <= 0) return 0;
+  for (int a = 1; a <= 8; a *= 2) {
+    if (p.tiles_n % a != 0 || p.tiles_m % (8 / a) != 0) continue;
+    const int64_t b_bytes = (int64_t)(p.tiles_n / a) * bn * p.K * 2;
+    if (b_bytes <= (5ll << 19)) return a;
+  }
+  return 0;
+}
+
 template <class Tile, bool PERM, int LAYOUT = 0>
 hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
   auto kernel = KernelOf<Tile, PERM, LAYOUT>::value;
@@ -149,6 +168,7 @@ hipError_t launch_kernel(const GemmParams& p_in, hipStream_t stream) {
   if constexpr (IsPersistent<Tile>::value) {
     const int cus = device_cus(dev);
     grid = dim3((unsigned)(total < cus ? total : cus), 1, 1);
+    p.xcd_cols = xcd_column_blocks(p, Tile::BN, (int)grid.x);
   }
   if constexpr (IsSplitK<Tile>::value) {
     // tiles are shared along K only with enough scratch memory to hold the partial tiles; without it the

@@ -58,6 +58,10 @@ struct GemmParams {
   void* ws;
   int64_t ws_bytes;
   int32_t split_k;  // number of workgroups that share a tile along K (set by the launcher of a split-K instance)
+  // Persistent kernels, one batch: when non-zero, XCD x owns the block of tiles_n / xcd_cols tile columns number
+  // x % xcd_cols and tiles_m * xcd_cols / 8 tile rows number x / xcd_cols, and walks it row by row (see
+  // map_tile_block).  Set by the launcher where the grid divides so and a block's B panels fit half an L2.
+  int32_t xcd_cols;
 };
 
 AITAMD_DEVICE int64_t out_batch_offset(const GemmParams& p, int batch) {

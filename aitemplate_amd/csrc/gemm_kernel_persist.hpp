@@ -173,7 +173,13 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     // virtual workgroup index: with one workgroup per CU, g % 8 is the XCD and stays it for every i
     int b, tm, tn;
     const bool half = split && i == full_rounds;
-    map_tile<8>(half ? full_rounds * G + split_tile : g + i * G, p.tiles_m, p.tiles_n, p.batch, b, tm, tn);
+    const int vwg = half ? full_rounds * G + split_tile : g + i * G;
+    if (p.xcd_cols > 0) {
+      b = 0;
+      map_tile_block(vwg, p.tiles_m, p.tiles_n, p.xcd_cols, tm, tn);
+    } else {
+      map_tile<8>(vwg, p.tiles_m, p.tiles_n, p.batch, b, tm, tn);
+    }
     c.m0 = tm * BM + (half ? split_half * (BM / 2) : 0);
     c.n0 = tn * BN;
     c.batch = b;
