@@ -28,6 +28,12 @@
 
 #include "common.hpp"
 
+#ifndef AITAMD_ATTN_FAST
+#define AITAMD_ATTN_FAST 1
+#endif
+#ifndef AITAMD_ATTN_BATCH_READS
+#define AITAMD_ATTN_BATCH_READS 0
+#endif
 #ifndef AITAMD_ATTN_KB
 #define AITAMD_ATTN_KB(KS, OT) (((KS) + 2 * (OT)) <= 7 ? 2 : 1)
 #endif
@@ -354,6 +360,9 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
     const float c = __builtin_fabsf(p.scale_log2e);
     float m_run = -INFINITY;
     float l_run = 0.0f;       // running sum over this lane's half of the keys
+#if AITAMD_ATTN_FAST
+    bool ref_ok = false;      // (wave-uniform) every row of the wave has a finite reference point
+#endif
 
     // wave-loads this wave issues per tile
     const int my_loads = (KL + VL - wave_ld + NWT - 1) / NWT;
@@ -428,6 +437,25 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         // (issuing the next block's product ahead of this block's softmax was measured: no gain at
         // head dim 40 and a quarter slower at head dim 64, where the extra live accumulator costs more)
         f32x16 s[KB];
+#if AITAMD_ATTN_BATCH_READS
+        // all K fragments of the block first, then its MFMAs: the reads overlap each other and the first MFMAs
+        // instead of each being waited for right behind its issue
+        {
+          vec8 kf[KB][KS];
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+              kf[kb][ks] = *reinterpret_cast<const vec8*>(cK + ((blk * KB + kb) * 32 + r32) * KPI + ks * 16 + h * 8);
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[kb][e] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) s[kb] = Tr::mfma32(kf[kb][ks], qf[ks], s[kb]);
+          }
+        }
+#else
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
 #pragma unroll
@@ -439,6 +467,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
             s[kb] = Tr::mfma32(kf, qf[ks], s[kb]);
           }
         }
+#endif
         // lane holds keys nb + 32 kb + 8 g + 4 h + r (element 4 g + r of sub-block kb) of query row q_row.
         // The running maximum is kept on the raw scores and the scale is folded into the exponent:
         // p = exp2(s * c - m * c) is one FMA and one v_exp per score (c > 0: a negative scale was moved into
@@ -495,10 +524,45 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           m_run = m_new;
         };
         const float m_before = m_run, l_before = l_run;
+#if AITAMD_ATTN_FAST
+        // Fast form of an unmasked block: no row maximum at all.  The probabilities are taken against the reference
+        // point the row already has, p = exp2((s - m) c); that is exact whatever m is, as long as no p leaves the
+        // element type's range, and a p beyond it shows as an infinite (or NaN) row sum, for which the block is
+        // redone below in the full form (maximum, moved reference point, rescaled accumulators).  After a row's
+        // first block - always the full form: there is no reference point yet - that takes a score 16 binary orders
+        // above everything the row has seen (fp16; never in practice for bf16), so nearly every block saves the
+        // maximum's 16 three-way compares, the exchange across the wave's halves and the bookkeeping of the
+        // reference point: 96 instead of 128 vector instructions per 64 keys.
+        bool full = need_mask || !ref_ok;
+        if (!full) {
+          const float mc = -m_run * c;
+#pragma unroll
+          for (int st = 0; st < 2 * KB; ++st) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const int kb = st >> 1, e = (st & 1) * 8 + j;
+              pf[st][j] = Tr::from_float(__builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][e], c, mc)));
+            }
+            l_run = add_elements(pf[st], l_run);
+          }
+          if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(l_run <= 3.0e38f)) != 0, 0)) {
+            l_run = l_before;
+            full = true;
+          }
+        }
+        if (full) {
+          if (need_mask)
+            softmax_block(std::true_type{}, std::false_type{});
+          else
+            softmax_block(std::false_type{}, std::false_type{});
+          ref_ok = __builtin_amdgcn_ballot_w64(__builtin_isinf(m_run)) == 0;
+        }
+#else
         if (need_mask)
           softmax_block(std::true_type{}, std::false_type{});
         else
           softmax_block(std::false_type{}, std::false_type{});
+#endif
         // A NaN score (a NaN in Q or in a K row) counts as -inf, i.e. its key is left out, as in the reference, whose
         // kernel applies ScaleAndResetNaNToMinusInfinity to the scores
         // (python/aitemplate/backend/rocm/gemm/bmm_softmax_bmm_permute.py:106, bmm_softmax_bmm.py:99).  The running
@@ -509,6 +573,9 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           m_run = m_before;
           l_run = l_before;
           softmax_block(std::true_type{}, std::true_type{});
+#if AITAMD_ATTN_FAST
+          ref_ok = __builtin_amdgcn_ballot_w64(__builtin_isinf(m_run)) == 0;
+#endif
         }
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
@@ -517,6 +584,29 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
             for (int e = 0; e < 16; ++e) oacc[ot][e] *= alpha;
         }
         // ---- O^T += V^T P^T over the block's 16-key steps
+#if AITAMD_ATTN_BATCH_READS
+        {
+          // all V^T fragments of the block first (the score registers are free by now), then the MFMAs
+          vec8 vfs[2 * KB][OT];
+#pragma unroll
+          for (int st = 0; st < 2 * KB; ++st)
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot) {
+              const T* vb = cV + (blk * KB * 32 + st * 16 + h * 4 + tr_row) * VPI + ((ot * 32) ^ tr_swz) + tr_col;
+              const vec4 lo = AttnVec<T>::tr_read(vb);
+              const vec4 hi = AttnVec<T>::tr_read(vb + 8 * VPI);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                vfs[st][ot][j] = lo[j];
+                vfs[st][ot][4 + j] = hi[j];
+              }
+            }
+#pragma unroll
+          for (int st = 0; st < 2 * KB; ++st)
+#pragma unroll
+            for (int ot = 0; ot < OT; ++ot) oacc[ot] = Tr::mfma32(vfs[st][ot], pf[st], oacc[ot]);
+        }
+#else
 #pragma unroll
         for (int st = 0; st < 2 * KB; ++st) {
 #pragma unroll
@@ -533,6 +623,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
             oacc[ot] = Tr::mfma32(vf, pf[st], oacc[ot]);
           }
         }
+#endif
       }
 
       if constexpr (!DMA) {

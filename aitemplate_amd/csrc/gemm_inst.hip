@@ -4,6 +4,7 @@
 // resulting launcher table under a C symbol the dispatcher looks up.
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 #include "gemm_host.hpp"
 #include "gemm_kernel_dma.hpp"
@@ -52,11 +53,22 @@ struct KernelOf<GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>, P
       gemm_rcr_dma_kernel<Elem, GemmTileDma<BM, BN, BK, WM, WN, NS, OCC, PIPE, MT, AUX, MODE>, Epi, PERM, LAYOUT>;
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int NS, int MT, int LBM, bool PERM, int LAYOUT>
-struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>, PERM, LAYOUT> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, int MT, int LBM, int PAIR, bool PERM, int LAYOUT>
+struct KernelOf<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM, PAIR>, PERM, LAYOUT> {
   // (LAYOUT 4 is not an operand layout: it names the instantiation for tiles of fewer K-slabs than ring stages)
   static constexpr auto value =
-      gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>, Epi, PERM, LAYOUT == kShortK>;
+      gemm_rcr_persist_kernel<Elem, GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM, PAIR>, Epi, PERM, LAYOUT == kShortK>;
+};
+// the slab-pair form of a persistent tile (the tile itself where it has none)
+template <class Tile>
+struct PairOf {
+  using type = Tile;
+};
+template <int BM, int BN, int BK, int WM, int WN, int MT, int LBM>
+struct PairOf<GemmTilePersist<BM, BN, BK, WM, WN, 4, MT, LBM, 0>> {
+  using Plain = GemmTilePersist<BM, BN, BK, WM, WN, 4, MT, LBM, 0>;
+  using type = std::conditional_t<Plain::kPairable,
+                                  GemmTilePersist<BM, BN, BK, WM, WN, 5, MT, LBM, Plain::kPairable ? 1 : 0>, Plain>;
 };
 // bit L set: the tile has a kernel for layout L (bit 0, rcr, always)
 template <class Tile>
@@ -87,8 +99,8 @@ template <class Tile>
 struct IsPersistent {
   static constexpr bool value = false;
 };
-template <int BM, int BN, int BK, int WM, int WN, int NS, int MT, int LBM>
-struct IsPersistent<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM>> {
+template <int BM, int BN, int BK, int WM, int WN, int NS, int MT, int LBM, int PAIR>
+struct IsPersistent<GemmTilePersist<BM, BN, BK, WM, WN, NS, MT, LBM, PAIR>> {
   static constexpr bool value = true;
 };
 
@@ -199,12 +211,27 @@ hipError_t launch_tile(const GemmParams& p, hipStream_t stream) {
     return hipErrorInvalidValue;
   }
   if constexpr (IsPersistent<Tile>::value) {
-    if ((p.K + Tile::BK - 1) / Tile::BK < Tile::NS) {
+    const int64_t k_tiles = ((int64_t)p.K + Tile::BK - 1) / Tile::BK;
+    if (k_tiles < Tile::NS) {
       if (p.perm_on) {
         if constexpr (kHasPermutedStore) return launch_kernel<Tile, true, kShortK>(p, stream);
         return hipErrorInvalidValue;
       }
       return launch_kernel<Tile, false, kShortK>(p, stream);
+    }
+    // tiles of an even number of K-slabs go to the slab-pair form of the kernel where the tile has one: the same
+    // products summed in the same order (the results are the same bit for bit), the loads better ordered
+    using Pair = typename PairOf<Tile>::type;
+    if constexpr (!std::is_same_v<Pair, Tile>) {
+      // (AITAMD_NO_SLAB_PAIRS=1 keeps every tile on the one-slab form, for measuring one against the other)
+      static const bool pairs_on = !(getenv("AITAMD_NO_SLAB_PAIRS") && atoi(getenv("AITAMD_NO_SLAB_PAIRS")) != 0);
+      if (pairs_on && k_tiles % 2 == 0 && k_tiles >= Tile::kPairMinSlabs) {
+        if (p.perm_on) {
+          if constexpr (kHasPermutedStore) return launch_kernel<Pair, true>(p, stream);
+          return hipErrorInvalidValue;
+        }
+        return launch_kernel<Pair, false>(p, stream);
+      }
     }
   }
   if (p.perm_on) {

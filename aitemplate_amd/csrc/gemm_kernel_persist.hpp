@@ -36,9 +36,14 @@ namespace aitamd {
 // LBM_: rows of the A slab a ring stage holds.  A tile of BM rows whose 16-row blocks do not divide over the waves
 // (224 rows: 14 blocks) takes the next size that does (256: rows past BM are cut off by the panel's buffer
 // descriptor - zero fill, nothing fetched - and no wave reads them).
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int MT_ = 32, int LBM_ = BM_>
+// PAIR_: the loader requests a K-slab and its successor together, 16 rows at a time (see the kernel): a row's two
+// 64-byte pieces are the halves of one 128-byte line of memory, and asked for back to back by one wave the second
+// finds the line in the CU's vector cache.  Needs a ring of five stages (two slabs can only be requested when two
+// stages are free), which leaves no room beside it: the epilogue's strips take the stage that is free then.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int NS_, int MT_ = 32, int LBM_ = BM_, int PAIR_ = 0>
 struct GemmTilePersist {
   static constexpr int LBM = LBM_;
+  static constexpr int PAIR = PAIR_;
   static constexpr int MT = MT_, KSTEP = MT == 32 ? 16 : 32, QN = 64 / MT, ACC_N = MT * MT / 64;
   static constexpr int BM = BM_, BN = BN_, BK = BK_;
   static constexpr int WGM = WGM_, WGN = WGN_, NS = NS_;
@@ -72,14 +77,25 @@ struct GemmTilePersist {
   static constexpr int STRIP_PITCH = WTN * 2;
   // rows of an epilogue strip pass: 32 (one or two block rows) where the LDS has room for it beside the ring
   // (and where a wave's rows are whole 32-row passes)
-  static constexpr int SB = (RING_BYTES + NW * 32 * STRIP_PITCH <= 160 * 1024 && WTM % 32 == 0) ? 32 : 16;
+  static constexpr bool kStripsFit32 =
+      PAIR ? NW * 32 * STRIP_PITCH <= STAGE_ELEMS * 2 : RING_BYTES + NW * 32 * STRIP_PITCH <= 160 * 1024;
+  static constexpr int SB = (kStripsFit32 && WTM % 32 == 0) ? 32 : 16;
   static constexpr int STRIP_BYTES = SB * STRIP_PITCH;
   static constexpr int ROWS_PER_PASS = 64 / STRIP_CHUNKS;
   static constexpr int PASSES = SB / ROWS_PER_PASS;
-  static constexpr int kLdsBytes = RING_BYTES + NW * STRIP_BYTES;
+  static constexpr int kLdsBytes = PAIR ? RING_BYTES : RING_BYTES + NW * STRIP_BYTES;
+  // a slab-pair form of this tile exists (five of its stages fit the LDS, its waves load four blocks each)
+  static constexpr bool kPairable = PAIR == 0 && MT == 16 && NS == 4 && BK == 32 && XTRA == 0 && L_MAIN == 4 &&
+      5 * STAGE_ELEMS * 2 <= 160 * 1024;
+  // fewest K-slabs per tile for which the launcher takes the slab-pair form (it needs an even number; below 16
+  // the longer fill and the peeled first pair cost what the loads gain: M=N=1000 K=256 0.0156 against 0.0150 ms)
+  static constexpr int kPairMinSlabs = 16;
   static_assert(MT == 32 || MT == 16, "MFMA block is 32x32 or 16x16");
   static_assert((MT == 32 && KK == 2) || (MT == 16 && KK == 1 && MI >= 2), "a slab is multiplied in two halves");
   static_assert(LBM >= BM && LBM % ROWS_PER_LOAD == 0, "the A slab in LDS holds the tile's rows");
+  static_assert(PAIR == 0 || (MT == 16 && NS == 5 && XTRA == 0 && L_MAIN == 4 && BK == 32 &&
+                              NW * STRIP_BYTES <= STAGE_ELEMS * 2),
+                "slab pairs: five stages of one-step slabs, four blocks per wave, the strips within one stage");
   static_assert(WTM % SB == 0, "a wave's rows are whole strip passes");
   static_assert(NS >= 4, "needs one slab in flight behind the one being waited for");
   static_assert(XTRA == 0 || (XTRA <= A_LOADS && NW % XTRA == 0 && L_P0 < LOADS_PER_STEP - 1),
@@ -116,7 +132,8 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
   const int wn = wave % Tile::WGN;
   const int fr = lane % MT;
   const int fq = lane / MT;
-  unsigned char* const strip = smem_raw + Tile::RING_BYTES + wave * Tile::STRIP_BYTES;
+  // (beside the ring; the slab-pair form moves it into the ring stage that is free during a tile's epilogue)
+  unsigned char* strip = smem_raw + (Tile::PAIR ? 0 : Tile::RING_BYTES) + wave * Tile::STRIP_BYTES;
 
   const int tiles_per_batch = p.tiles_m * p.tiles_n;
   const int total_tiles = tiles_per_batch * p.batch;
@@ -569,6 +586,188 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
     }
     wait_vmcnt<0>();
     return;
+  } else if constexpr (Tile::PAIR != 0) {
+    // ---- slab pairs ---------------------------------------------------------------------------------------
+    // The K loop in units of two slabs (a, b), a even.  Multiplying is as in the loop below - every slab in two
+    // halves around its barrier, the first fetching the lower A rows of its slab from LDS, the second the next
+    // slab's upper A rows and B fragments (B alternates between two register sets, so these go out at the start
+    // of the half, not as the last MFMAs release the registers).  Loading differs: a wave requests block i of
+    // slab a' and block i of slab b' back to back - the same 16 rows, the two 64-byte halves of the same lines.
+    // Measured with the loads alone (no MFMAs, constant operands), such pairs against one slab at a time:
+    // M=N=8192 K=8192 0.67 against 0.73 ms, M=24576 N=3072 K=768 0.069 against 0.090 ms.
+    // With slab t in ring stage t % 5, the two stages of the pair (a + 4, a + 5) are both free behind a's barrier
+    // (a's own stage and that of the slab before it).  A wave requests its four blocks of that pair one per half
+    // slab - second half of a, both halves of b, first half of a + 2 - so every half issues two loads, as in the
+    // loop below, and a load has one to three slab times to arrive.  Which tile a request belongs to is a scalar
+    // select per pair, so one loop body serves the whole K range of a tile and the hand-over to the next one.
+    // Needs tiles of an even number of slabs, at least four.
+    struct Panel {
+      uint32_t lo, hi, bytes;
+    };
+    auto tile_panel = [&](int i) __attribute__((always_inline)) {
+      Panel q;
+      const void* base = p.a;
+      uint32_t bytes = 0;
+      if (i < my_tiles) {
+        const TileCoord c = tile_coord(i);
+        const int rows_a = (p.M - c.m0) < c.rows ? (p.M - c.m0) : c.rows;
+        const int rows_b = (p.N - c.n0) < BN ? (p.N - c.n0) : BN;
+        const T* Ab = reinterpret_cast<const T*>(p.a) + (int64_t)c.batch * p.sa + (int64_t)c.m0 * p.lda;
+        const T* Bb = reinterpret_cast<const T*>(p.b) + (int64_t)c.batch * p.sb + (int64_t)c.n0 * p.ldb;
+        const uint32_t bytes_a = rows_a > 0 ? clamp_records((((int64_t)rows_a - 1) * p.lda + p.K) * 2) : 0u;
+        const uint32_t bytes_b = clamp_records((((int64_t)rows_b - 1) * p.ldb + p.K) * 2);
+        base = loads_a ? (const void*)Ab : (const void*)Bb;
+        bytes = loads_a ? bytes_a : bytes_b;
+      }
+      const uint64_t v = reinterpret_cast<uint64_t>(base);
+      q.lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+      q.hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+      q.bytes = __builtin_amdgcn_readfirstlane(bytes);
+      return q;
+    };
+    auto panel_rsrc = [&](const Panel& q) __attribute__((always_inline)) {
+      return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((uint64_t)q.hi << 32) | q.lo), 0, q.bytes,
+                                               0x00020000);
+    };
+    // byte offset of the lane's chunk in block i of the wave (every load has its own LDS base here)
+    uint32_t lp_off[L];
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+      const int j = wave * LM + i;
+      const int row = (loads_a ? j : j - Tile::A_MAIN) * Tile::ROWS_PER_LOAD + l_row;
+      lp_off[i] = (uint32_t)(((int64_t)row * (loads_a ? p.lda : p.ldb) + l_chunk_k[i]) * 2);
+    }
+    auto ring_stage = [&](int st) __attribute__((always_inline)) { return smem + st * Tile::STAGE_ELEMS; };
+    auto wrap = [](int st) __attribute__((always_inline)) { return st >= NS ? st - NS : st; };
+    // blocks [I0, I1) of the wave for the slabs kt (even) and kt + 1 of the tile behind d, into stages sa_ and sb_
+    auto issue_pair = [&](auto i0_c, auto i1_c, const __amdgpu_buffer_rsrc_t& d, int kt, int sa_, int sb_)
+                          __attribute__((always_inline)) {
+      constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
+      const int k0 = kt * BK;
+      static_for<I0, I1>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        const uint32_t off_a = (k0 + l_chunk_k[i] < p.K) ? lp_off[i] + (uint32_t)(k0 * 2) : kOobOffset;
+        const uint32_t off_b = (k0 + BK + l_chunk_k[i] < p.K) ? lp_off[i] + (uint32_t)((k0 + BK) * 2) : kOobOffset;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (lds_void*)(ring_stage(sa_) + (l_block0 + i) * 512), 16, off_a, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(d, (lds_void*)(ring_stage(sb_) + (l_block0 + i) * 512), 16, off_b, 0, 0, 0);
+      });
+    };
+    constexpr std::integral_constant<int, 0> b_0{};
+    constexpr std::integral_constant<int, 1> b_1{};
+    constexpr std::integral_constant<int, 2> b_2{};
+    constexpr std::integral_constant<int, 3> b_3{};
+    constexpr std::integral_constant<int, 4> b_4{};
+    static_assert(L == 4, "four blocks per wave, one per half slab of a pair");
+    Panel cur_p = tile_panel(0), nxt_p = cur_p;
+    // prologue: pair 0 whole and blocks 0 to 2 of pair 1 (what the three halves before the loop would have
+    // requested); slab 0 has landed when only its successor's last block and pair 1's six loads are outstanding
+    {
+      const __amdgpu_buffer_rsrc_t d0 = panel_rsrc(cur_p);
+      issue_pair(b_0, b_4, d0, 0, 0, 1);
+      issue_pair(b_0, b_3, d0, 2, 2, 3);
+      wait_vmcnt<7>();
+      __builtin_amdgcn_s_barrier();
+    }
+    vec8 bfn[NI];  // B fragments of a pair's second slab
+    load_a(smem, 0, af[0]);
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) bf[0][ni] = load_b1(smem, 0, ni);
+    int sa = 0;  // ring stage of the pair's first slab
+
+    // One pair in stages sa, sa + 1.  (p1, kt1): panel and first slab of the next pair (its block 3 goes out in the
+    // first half of a); (p2, kt2): of the pair after that (blocks 0 to 2, in the three halves behind a's barrier).
+    auto pair = [&](auto active_c, auto first_c, const Panel& p1, int kt1, const Panel& p2, int kt2) __attribute__((always_inline)) {
+      constexpr bool ACTIVE = decltype(active_c)::value;
+      constexpr bool FIRST = decltype(first_c)::value;  // the tile's first pair: slab a starts the accumulators
+      const int s1 = wrap(sa + 1), s2 = wrap(sa + 2), s3 = wrap(sa + 3), s4 = wrap(sa + 4);
+      const T* st_a = ring_stage(sa);
+      const T* st_b = ring_stage(s1);
+      const T* st_n = ring_stage(s2);
+      const __amdgpu_buffer_rsrc_t d2 = panel_rsrc(p2);
+      // first half of a
+      issue_pair(b_3, b_4, panel_rsrc(p1), kt1, s2, s3);
+      if constexpr (ACTIVE) {
+        load_a(st_a, 1, af[1]);
+        if constexpr (FIRST)
+          mfmas_first(af[0], bf[0]);
+        else
+          mfmas(af[0], bf[0]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // slab b has landed: only the eight loads of the four halves since its last block are younger.  The LDS reads
+      // of a are waited for as well (they were issued a half slab ago): a's stage is written to behind the barrier.
+      __builtin_amdgcn_s_waitcnt((8 & 0xf) | (0x7 << 4) | (0 << 8));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // second half of a
+      issue_pair(b_0, b_1, d2, kt2, s4, sa);
+      if constexpr (ACTIVE) {
+        load_a(st_b, 0, af[0]);
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) bfn[ni] = load_b1(st_b, 0, ni);
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+          for (int mi = 0; mi < MH2; ++mi)
+            acc[MH + mi][ni] = Mfma::run(bf[0][ni], af[1][mi], FIRST ? acc_t{} : acc[MH + mi][ni]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // first half of b
+      issue_pair(b_1, b_2, d2, kt2, s4, sa);
+      if constexpr (ACTIVE) {
+        load_a(st_b, 1, af[1]);
+        mfmas(af[0], bfn);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      wait_vmcnt<5>();  // the next pair's first slab has landed: younger are its last block's other half and two blocks
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // second half of b
+      issue_pair(b_2, b_3, d2, kt2, s4, sa);
+      if constexpr (ACTIVE) {
+        load_a(st_n, 0, af[0]);
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) bf[0][ni] = load_b1(st_n, 0, ni);
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+          for (int mi = 0; mi < MH2; ++mi) acc[MH + mi][ni] = Mfma::run(bfn[ni], af[1][mi], acc[MH + mi][ni]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      sa = s2;
+    };
+    const int n_pairs = k_tiles / 2;  // (the launcher checks: an even number of slabs, at least four)
+    auto tile_pairs = [&](auto active_c) __attribute__((always_inline)) {
+      auto one = [&](auto first_c, int j) __attribute__((always_inline)) {
+        const bool in1 = j + 1 < n_pairs, in2 = j + 2 < n_pairs;
+        Panel p1, p2;
+        p1.lo = in1 ? cur_p.lo : nxt_p.lo;
+        p1.hi = in1 ? cur_p.hi : nxt_p.hi;
+        p1.bytes = in1 ? cur_p.bytes : nxt_p.bytes;
+        p2.lo = in2 ? cur_p.lo : nxt_p.lo;
+        p2.hi = in2 ? cur_p.hi : nxt_p.hi;
+        p2.bytes = in2 ? cur_p.bytes : nxt_p.bytes;
+        pair(active_c, first_c, p1, in1 ? 2 * j + 2 : 0, p2, in2 ? 2 * j + 4 : 2 * (j + 2 - n_pairs));
+      };
+      one(std::true_type{}, 0);
+      for (int j = 1; j < n_pairs; ++j) one(std::false_type{}, j);
+    };
+    for (int i = 0; i < my_tiles; ++i) {
+      const TileCoord cur = tile_coord(i);
+      nxt_p = tile_panel(i + 1);
+      const bool active = wm * Tile::WTM < cur.rows;
+      if (active) {
+        tile_pairs(std::true_type{});
+        // the stage of the tile's last slab is free until the next tile's first slab has passed its barrier, which
+        // no wave reaches before every wave has left this epilogue
+        strip = smem_raw + wrap(sa + NS - 1) * (Tile::STAGE_ELEMS * 2) + wave * Tile::STRIP_BYTES;
+        epilogue(cur);
+      } else {
+        tile_pairs(std::false_type{});
+      }
+      cur_p = nxt_p;
+    }
+    wait_vmcnt<0>();
   } else {
   // prologue: slabs 0 .. NS-3 whole, slab NS-2 up to its first portion
 #pragma unroll

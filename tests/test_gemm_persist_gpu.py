@@ -1,7 +1,8 @@
 """GPU parity of the persistent GEMM instances (one workgroup per CU walks its tiles, the LDS ring
 runs across tile boundaries): many tiles per workgroup, fewer tiles than CUs, single-slab K, K
 tails, M/N tails, the scalar-store path (N not a multiple of 8), strided views, batches, bf16,
-every epilogue."""
+every epilogue.  Tiles of an even number of K-slabs, 16 or more, run the slab-pair form of the kernel
+where the instance has one: the shapes below cover both forms and the switch between them."""
 import pytest
 import torch
 
@@ -69,6 +70,12 @@ def test_persist_instances_exist():
     (4000, 4352, 64),    # 272 tiles on 256 CUs: the 16 leftover tiles are split in halves; M tail of 160 rows
     (3900, 4352, 64),    # same, M tail of 60 rows: some lower halves lie wholly below M
     (24576, 768, 128),   # 288 tiles: one full round plus 32 split tiles
+    (1000, 392, 512),    # 16 slabs: the shortest tile of the slab-pair form
+    (515, 264, 1000),    # 32 slabs, the last one ragged (K tail inside a pair)
+    (300, 264, 520),     # 17 slabs: odd, the one-slab form
+    (4000, 4352, 576),   # 18 slabs, 272 tiles: pairs across tile boundaries, leftover tiles split in halves
+    (3900, 4352, 512),   # same with lower halves wholly below M (waves that load but do not multiply)
+    (2048, 1536, 2048),  # 48 tiles of 64 slabs
 ])
 def test_persist_shapes(name, shape):
     M, N, K = shape
@@ -80,6 +87,7 @@ def test_persist_shapes(name, shape):
 @pytest.mark.parametrize("op", sorted(set(_kernels.EPILOGUE_OF_OP) - {"bmm_rcr"}))
 def test_persist_every_epilogue(name, op):
     _check(op, name, 1000, 392, 320, seed=7)
+    _check(op, name, 1000, 392, 640, seed=8)   # 20 slabs: the slab-pair form
 
 
 @pytest.mark.parametrize("name", _persist_names())
@@ -87,6 +95,7 @@ def test_persist_scalar_store_path(name):
     # N not a multiple of 8 -> element-wise stores and bias reads
     _check("gemm_rcr_bias_gelu", name, 333, 100, 64, seed=3)
     _check("gemm_rcr_bias_add", name, 700, 250, 160, seed=4)
+    _check("gemm_rcr_bias_add", name, 700, 250, 1024, seed=5)
 
 
 @pytest.mark.parametrize("name", _persist_names())
