@@ -143,8 +143,13 @@ AITAMD_DEVICE uint32_t clamp_records(int64_t bytes) {
 // L2 only.  Step 1 gives every XCD a contiguous range of logical (batch, tile) ids,
 // step 2 walks the tiles of a batch in groups of kGroupM tile-rows, column by column.
 // ---------------------------------------------------------------------------
+AITAMD_DEVICE void map_tile_grouped(int wg, int tiles_m, int tiles_n, int batch, int kGroupM, int& b, int& tm, int& tn);
 template <int kGroupM>
 AITAMD_DEVICE void map_tile(int wg, int tiles_m, int tiles_n, int batch, int& b, int& tm, int& tn) {
+  map_tile_grouped(wg, tiles_m, tiles_n, batch, kGroupM, b, tm, tn);
+}
+// (the group height as a value: the persistent kernels take it from the launcher)
+AITAMD_DEVICE void map_tile_grouped(int wg, int tiles_m, int tiles_n, int batch, int kGroupM, int& b, int& tm, int& tn) {
   // wg runs over batch * tiles_m * tiles_n workgroups; logical ids are batch-major, so an XCD's
   // contiguous id range is a run of whole batches (plus at most two partial ones at its ends):
   // the tiles of one batch share its operands through one L2 and fill its output rows together.

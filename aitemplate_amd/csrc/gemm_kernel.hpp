@@ -62,6 +62,9 @@ struct GemmParams {
   // x % xcd_cols and tiles_m * xcd_cols / 8 tile rows number x / xcd_cols, and walks it row by row (see
   // map_tile_block).  Set by the launcher where the grid divides so and a block's B panels fit half an L2.
   int32_t xcd_cols;
+  // Persistent kernels without the block mapping: tile rows per group of the grouped walk (0: eight).  An XCD's run
+  // of consecutive tiles is walked group by group, column by column inside a group.
+  int32_t group_m;
 };
 
 AITAMD_DEVICE int64_t out_batch_offset(const GemmParams& p, int batch) {

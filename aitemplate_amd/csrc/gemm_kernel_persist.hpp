@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
       b = 0;
       map_tile_block(vwg, p.tiles_m, p.tiles_n, p.xcd_cols, tm, tn);
     } else {
-      map_tile<8>(vwg, p.tiles_m, p.tiles_n, p.batch, b, tm, tn);
+      map_tile_grouped(vwg, p.tiles_m, p.tiles_n, p.batch, p.group_m > 0 ? p.group_m : 8, b, tm, tn);
     }
     c.m0 = tm * BM + (half ? split_half * (BM / 2) : 0);
     c.n0 = tn * BN;

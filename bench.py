@@ -26,13 +26,28 @@ if ROOT not in sys.path:
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the headline workload, per kernel instance: (bytes, the file under profiles/ that holds
-# the two counter runs of this script the figure comes from: FETCH_SIZE, then WRITE_SIZE, each scaled by what the
-# same counter read for the 256 MiB copy of --copy-probe in the same run).  An instance that is not listed was
-# never measured and reports null with that reason.
+# HBM bytes per launch, per (configuration, kernel instance): (bytes, the file under profiles/ that holds the two
+# counter runs of this script the figure comes from: FETCH_SIZE, then WRITE_SIZE, each scaled by what the same
+# counter read for the 256 MiB copy of --copy-probe in the same run).  A pair that is not listed was never measured
+# and reports null with that reason.
 MEASURED_TRAFFIC = {
-    "gemm_rcr_f16_256x256x32_w2x4_persist4_m16": (331_374_000, "profiles/gemm_rcr_persist_kernel_bias_gelu_M24576_N3072_K768_counters.txt"),
+    ("c2a", "gemm_rcr_f16_256x256x32_w2x4_persist4_m16"):
+        (320_584_000, "profiles/gemm_rcr_persist_kernel_bias_gelu_M24576_N3072_K768_counters.txt"),
+    ("c2b", "gemm_rcr_f16_320x256x32_w2x4_persist4_m16"):
+        (307_647_000, "profiles/gemm_rcr_persist_kernel_bias_add_M24576_N768_K3072.txt"),
+    ("c3", "gemm_rcr_f16_224x256x32_w2x4_persist4_m16"):
+        (253_676_000, "profiles/gemm_rcr_persist_kernel_bias_add_add_M12608_N1024_K4096.txt"),
+    ("c1", "gemm_rcr_f16_32x32x128_w2x2_dma4_o2_p0_m16_c0"):
+        (6_892_000, "profiles/gemm_rcr_dma_kernel_bias_M256_N1024_K1024.txt"),
 }
+
+
+def measured_traffic(workload, instance):
+    """(bytes or None, where the figure comes from or why there is none)."""
+    t = MEASURED_TRAFFIC.get((workload, instance))
+    if t is None:
+        return None, f"no counter run of instance {instance} on configuration {workload} is held under profiles/"
+    return t[0], f"{t[1]} (instance {instance})"
 
 SHAPES = {
     # name: (op, M, N, K, residuals)
@@ -253,6 +268,8 @@ def other_configs(torch, eager, kernels, steps, warmup, vendor_baseline=True):
                      "ms": round(r["event_ms_per_launch"], 5), "median_ms": round(r["median_ms_per_launch"], 5),
                      "tflops": round(case.flops / r["event_ms_per_launch"] / 1e9, 2),
                      "roofline": _roofline("mfma", case.flops, r["event_ms_per_launch"], r["median_ms_per_launch"])}
+        out[name]["roofline"]["traffic"], out[name]["roofline"]["traffic_source"] = measured_traffic(
+            name, out[name]["instance"])
         if vendor_baseline:
             # a baseline, not part of the product: the same result from PyTorch-ROCm's own operators on the same
             # operand sets (its GEMM library with a bias, then one add kernel per residual)
@@ -476,10 +493,7 @@ def main():
     roofline["median_launch_ms"] = round(r["median_ms_per_launch"], 5)
     roofline["median_of"] = f"{r['groups']} groups of consecutive launches inside the timed region"
     roofline["settle_launches"] = r["settle_launches"]
-    traffic = MEASURED_TRAFFIC.get(instance)
-    roofline["traffic"] = traffic[0] if traffic else None
-    roofline["traffic_source"] = (f"{traffic[1]} (instance {instance})" if traffic else
-                                  f"no counter run of instance {instance} is held under profiles/")
+    roofline["traffic"], roofline["traffic_source"] = measured_traffic(args.workload, instance)
     # The device is power-limited on this kernel and its engine clock follows the operands: the same launch on
     # constant data (no toggling in the multipliers) is a diagnostic for how much of the distance to the peak is
     # clock, not schedule.  Never the reported value.

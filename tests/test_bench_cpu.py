@@ -47,11 +47,17 @@ def test_power_sampler_without_a_sensor_reports_nothing(tmp_path):
 
 
 def test_traffic_table_names_files_that_exist():
-    for instance, (nbytes, path) in bench.MEASURED_TRAFFIC.items():
+    for (workload, instance), (nbytes, path) in bench.MEASURED_TRAFFIC.items():
+        assert workload in bench.SHAPES
         assert nbytes > 0
         full = os.path.join(ROOT, path)
         assert os.path.isfile(full), path
-        assert instance in open(full).read()
+        text = open(full).read()
+        assert instance in text
+        # the file shows the figure itself, as megabytes or written out
+        assert f"{nbytes:,}".replace(",", " ") in text, (path, nbytes)
+        assert bench.measured_traffic(workload, instance)[0] == nbytes
+    assert bench.measured_traffic("c2a", "no_such_instance")[0] is None
 
 
 def test_graph_of_a_launch_bound_configuration_never_holds_fewer_than_100_launches():
