@@ -693,12 +693,10 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
         else
           mfmas(af[0], bf[0]);
       }
-      __builtin_amdgcn_sched_barrier(0);
       // slab b has landed: only the eight loads of the four halves since its last block are younger.  The LDS reads
       // of a are waited for as well (they were issued a half slab ago): a's stage is written to behind the barrier.
       __builtin_amdgcn_s_waitcnt((8 & 0xf) | (0x7 << 4) | (0 << 8));
       __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
       // second half of a
       issue_pair(b_0, b_1, d2, kt2, s4, sa);
       if constexpr (ACTIVE) {
@@ -711,17 +709,14 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
           for (int mi = 0; mi < MH2; ++mi)
             acc[MH + mi][ni] = Mfma::run(bf[0][ni], af[1][mi], FIRST ? acc_t{} : acc[MH + mi][ni]);
       }
-      __builtin_amdgcn_sched_barrier(0);
       // first half of b
       issue_pair(b_1, b_2, d2, kt2, s4, sa);
       if constexpr (ACTIVE) {
         load_a(st_b, 1, af[1]);
         mfmas(af[0], bfn);
       }
-      __builtin_amdgcn_sched_barrier(0);
       wait_vmcnt<5>();  // the next pair's first slab has landed: younger are its last block's other half and two blocks
       __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
       // second half of b
       issue_pair(b_2, b_3, d2, kt2, s4, sa);
       if constexpr (ACTIVE) {
@@ -733,7 +728,6 @@ __global__ void __launch_bounds__(Tile::NT, 1) gemm_rcr_persist_kernel(const Gem
 #pragma unroll
           for (int mi = 0; mi < MH2; ++mi) acc[MH + mi][ni] = Mfma::run(bfn[ni], af[1][mi], acc[MH + mi][ni]);
       }
-      __builtin_amdgcn_sched_barrier(0);
       sa = s2;
     };
     const int n_pairs = k_tiles / 2;  // (the launcher checks: an even number of slabs, at least four)
