@@ -102,11 +102,19 @@ struct AttnVec<f16> {
     const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((__attribute__((address_space(3))) raw4*)p);
     return __builtin_bit_cast(f16x4, r);
   }
+  static AITAMD_DEVICE f16x4 tr_read(__attribute__((address_space(3))) const f16* p) {
+    const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((__attribute__((address_space(3))) raw4*)p);
+    return __builtin_bit_cast(f16x4, r);
+  }
 };
 template <>
 struct AttnVec<bf16> {
   typedef __bf16 raw4 __attribute__((__vector_size__(4 * sizeof(__bf16))));
   static AITAMD_DEVICE bf16x4 tr_read(const bf16* p) {
+    const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) raw4*)p);
+    return __builtin_bit_cast(bf16x4, r);
+  }
+  static AITAMD_DEVICE bf16x4 tr_read(__attribute__((address_space(3))) const bf16* p) {
     const raw4 r = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) raw4*)p);
     return __builtin_bit_cast(bf16x4, r);
   }
@@ -429,6 +437,19 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
       }
       const T* cK = sK + cur * BN * KPI;
       const T* cV = sV + cur * BN * VPI;
+      // The lane's LDS addresses of the tile, one per operand (and per 32-column block of V, whose swizzle sits
+      // in the column bits), taken once per tile and made opaque: every fragment read of the tile is then that
+      // register plus an immediate offset.  Left to itself the compiler re-adds stage base, lane offset and block
+      // offset in front of every read (22 vector instructions per 64 keys).
+      typedef __attribute__((address_space(3))) const T lds_T;
+      lds_T* k_lane = (lds_T*)(cK + r32 * KPI + h * 8);
+      asm volatile("" : "+v"(k_lane));
+      lds_T* v_lane[OT];
+#pragma unroll
+      for (int ot = 0; ot < OT; ++ot) {
+        v_lane[ot] = (lds_T*)(cV + (h * 4 + tr_row) * VPI + ((ot * 32) ^ tr_swz) + tr_col);
+        asm volatile("" : "+v"(v_lane[ot]));
+      }
 
 #pragma unroll
       for (int blk = 0; blk < BN / (32 * KB); ++blk) {
@@ -462,8 +483,8 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
           for (int e = 0; e < 16; ++e) s[kb][e] = 0.0f;
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
-            const vec8 kf =
-                *reinterpret_cast<const vec8*>(cK + ((blk * KB + kb) * 32 + r32) * KPI + ks * 16 + h * 8);
+            typedef __attribute__((address_space(3))) const vec8 lds_vec8;
+            const vec8 kf = *(lds_vec8*)(k_lane + (blk * KB + kb) * 32 * KPI + ks * 16);
             s[kb] = Tr::mfma32(kf, qf[ks], s[kb]);
           }
         }
@@ -611,7 +632,7 @@ __global__ void __launch_bounds__(Tile::NT, Tile::NW == 4 ? 2 : 1) attention_ker
         for (int st = 0; st < 2 * KB; ++st) {
 #pragma unroll
           for (int ot = 0; ot < OT; ++ot) {
-            const T* vb = cV + (blk * KB * 32 + st * 16 + h * 4 + tr_row) * VPI + ((ot * 32) ^ tr_swz) + tr_col;
+            lds_T* vb = v_lane[ot] + (blk * KB * 32 + st * 16) * VPI;
             const vec4 lo = AttnVec<T>::tr_read(vb);
             const vec4 hi = AttnVec<T>::tr_read(vb + 8 * VPI);
             vec8 vf;
