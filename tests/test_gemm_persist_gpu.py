@@ -122,6 +122,21 @@ def test_persist_bmm_batches_and_views(name):
     got = eager.bmm_rcr(a, b, algo=_algo("gemm_rcr", name))
     torch.cuda.synchronize()
     torch.testing.assert_close(got.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    # the same with 18 K-slabs per tile: the slab-pair form, pairs handed over from one batch entry to the next
+    a = _rand((5, 300, 576), torch.float16, 3, 0.25).cuda()
+    b = _rand((5, 264, 576), torch.float16, 4, 0.25).cuda()
+    want = oracle.torch_bmm_rcr(a.cpu(), b.cpu()).half().float()
+    got = eager.bmm_rcr(a, b, algo=_algo("gemm_rcr", name))
+    torch.cuda.synchronize()
+    torch.testing.assert_close(got.cpu().float(), want, atol=1e-2, rtol=1e-2)
+    wide = _rand((300, 2048), torch.float16, 8).cuda()
+    xv = wide[:, 256:256 + 1024]                 # row pitch 2048, offset 256, 32 slabs
+    wv = _rand((264, 1024), torch.float16, 9, 1024 ** -0.5).cuda()
+    bv = _rand((264,), torch.float16, 10).cuda()
+    want = oracle.torch_gemm("gemm_rcr_bias", xv.cpu(), wv.cpu(), bv.cpu()).half().float()
+    got = eager.gemm("gemm_rcr_bias", xv, wv, bv, algo=_algo("gemm_rcr_bias", name))
+    torch.cuda.synchronize()
+    torch.testing.assert_close(got.cpu().float(), want, atol=1e-2, rtol=1e-2)
     big = _rand((500, 512), torch.float16, 5).cuda()
     x = big[:, 64:64 + 256]                      # row pitch 512, offset 64
     w = _rand((264, 256), torch.float16, 6, 256 ** -0.5).cuda()
