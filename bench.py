@@ -116,8 +116,11 @@ class PowerSampler:
                 "source": f"{os.path.basename(self.path)} of the card's hwmon, every 20 ms over the last 60 % of the region"}
 
 
-SETTLE_LAUNCHES = 400      # untimed launches in front of every timed region, whatever --warmup says
+# untimed launches in front of every timed region, whatever --warmup says (AITAMD_BENCH_SETTLE overrides: a knob for
+# measuring how long the clocks take to settle, not for the metric)
+SETTLE_LAUNCHES = int(os.environ.get("AITAMD_BENCH_SETTLE", "400"))
 GRAPH_MIN_LAUNCHES = 100   # launches held by the graph a launch-bound configuration is timed with
+MIN_GROUP_LAUNCHES = 10    # fewest direct launches between two of the events that cut a timed region into groups
 
 
 def graph_plan(steps, groups, min_launches=GRAPH_MIN_LAUNCHES):
@@ -140,7 +143,10 @@ def timed_region(torch, step, steps, warmup, groups=20, graph=False, power=None,
     for i in range(settle + warmup):
         step(i)
     torch.cuda.synchronize()
-    groups = max(1, min(groups, steps))
+    # a group holds at least MIN_GROUP_LAUNCHES launches: an event between two launches keeps the second from
+    # starting while the first one's last workgroups finish, 3 to 4 us per launch of the headline kernel (measured:
+    # 20 steps in 20 groups 0.1265-0.1305 ms per launch, in the same process 1000 steps in 20 groups 0.1230-0.1241)
+    groups = max(1, min(groups, steps // MIN_GROUP_LAUNCHES if not graph else steps))
     cuts = [steps * g // groups for g in range(groups + 1)]
     if graph:
         per, groups = graph_plan(steps, groups)

@@ -102,6 +102,7 @@ def test_timed_region_runs_settle_and_warmup_untimed_and_times_exactly_k_steps()
     _FakeTorch.cuda.issued = 0
     r = bench.timed_region(_FakeTorch, step, 20, 5, settle=300)
     assert len(calls) == 300 + 5 + 20
-    assert r["steps"] == 20 and r["settle_launches"] == 300 and r["groups"] == 20
+    # the driver's 20 steps make two groups of ten: no event between single launches
+    assert r["steps"] == 20 and r["settle_launches"] == 300 and r["groups"] == 2
     assert r["event_ms_per_launch"] == 1.0 and r["median_ms_per_launch"] == 1.0  # one "ms" per fake launch
     assert bench.SETTLE_LAUNCHES >= 300
